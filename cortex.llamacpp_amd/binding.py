@@ -8,6 +8,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K = 0, 1, 2, 8, 12, 13, 14, 15
+BF16 = 30
 Q2_K, Q3_K = 10, 11
 Q5_0, IQ4_NL = 6, 20
 
@@ -29,7 +30,7 @@ class ModelParams(C.Structure):
 class ContextParams(C.Structure):
     _fields_ = [("n_ctx", C.c_uint32), ("n_batch", C.c_uint32), ("n_ubatch", C.c_uint32), ("n_seq_max", C.c_uint32),
                 ("type_k", C.c_int32), ("type_v", C.c_int32), ("flash_attn", C.c_int32), ("embeddings", C.c_int32),
-                ("use_graphs", C.c_int32), ("logits_to_host", C.c_int32)]
+                ("use_graphs", C.c_int32), ("logits_to_host", C.c_int32), ("exact_f32", C.c_int32)]
 
 
 class Batch(C.Structure):
@@ -542,13 +543,14 @@ class Model:
 class Context:
     def __init__(self, model: Model, n_ctx: int = 512, n_batch: int = 2048, n_ubatch: int = 512, n_seq_max: int = 1,
                  type_k: int = F16, type_v: int = F16, flash_attn: bool = True, use_graphs: bool = True,
-                 logits_to_host: bool = True):
+                 logits_to_host: bool = True, exact_f32: bool = False):
         self.lib = model.lib
         self.model = model
         cp = self.lib.mi355_context_default_params()
         cp.n_ctx, cp.n_batch, cp.n_ubatch, cp.n_seq_max = n_ctx, n_batch, n_ubatch, n_seq_max
         cp.type_k, cp.type_v, cp.flash_attn, cp.use_graphs = type_k, type_v, int(flash_attn), int(use_graphs)
         cp.logits_to_host = int(logits_to_host)
+        cp.exact_f32 = int(exact_f32)
         self.h = self.lib.mi355_context_new(model.h, cp)
         if not self.h:
             raise MI355Error(f"mi355_context_new failed: {_err(self.lib)}")

@@ -254,6 +254,43 @@ hipError_t launch_add(const float *a, const float *b, float *y, int64_t n, hipSt
     return hipGetLastError();
 }
 
+// RMS norm of f32 rows kept in f32 end to end, for layers that put a norm on both sides of a sublayer:  y = [resid +] x / sqrt(mean(x^2) + eps) * (w_off + w).
+// w_off 1: zero-centred weights (the file holds w, the factor is 1 + w); resid == y adds the normed sublayer output into the residual stream in place.  Any n; the root and the division are
+// the correctly rounded ones (no reciprocal-square-root approximation).
+__global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float *__restrict__ x, int ld_x, const float *__restrict__ w, float w_off, const float *resid, float *y, int ld_y,
+                                                          int n, float eps) {
+    __shared__ float part[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float *xr = x + (size_t)t * ld_x;
+    float ss = 0.0f;
+    for (int i = tid; i < n; i += 256) { const float v = xr[i]; ss = fmaf(v, v, ss); }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if ((tid & 63) == 0) part[tid >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)n + eps);
+    for (int i = tid; i < n; i += 256) {
+        const float v = xr[i] * inv * (w_off + w[i]);
+        y[(size_t)t * ld_y + i] = resid ? resid[(size_t)t * ld_y + i] + v : v;
+    }
+}
+hipError_t launch_rmsnorm_f32(const float *x, int ld_x, const float *w, float w_off, const float *resid, float *y, int ld_y, int n, int T, float eps, hipStream_t st) {
+    if (T <= 0 || n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(rmsnorm_f32_kernel, dim3((unsigned)T), dim3(256), 0, st, x, ld_x, w, w_off, resid, y, ld_y, n, eps);
+    return hipGetLastError();
+}
+// x[t][i] += row[i] for T rows of n
+__global__ void add_row_kernel(float *x, const float *row, int n, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] += row[i % n];
+}
+hipError_t launch_add_row(float *x, const float *row, int n, int T, hipStream_t st) {
+    const int64_t total = (int64_t)n * T;
+    if (total <= 0) return hipSuccess;
+    hipLaunchKernelGGL(add_row_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, x, row, n, total);
+    return hipGetLastError();
+}
+
 // the Q / K / V bias vectors of a qwen2-style attention block added to all T rows of the three projections in one launch (a null bias skips its segment);
 // grid.y = 0, 1, 2 picks the projection
 __global__ void add_qkv_bias_kernel(float *q, float *k, float *v, const float *bq, const float *bk, const float *bv, int nq, int nkv, int T) {

@@ -153,7 +153,7 @@ int mi355_model_meta_str(const mi355_model *m, const char *key, char *buf, size_
 mi355_context_params mi355_context_default_params(void) {
     mi355_context_params p{};
     p.n_ctx = 2048; p.n_batch = 2048; p.n_ubatch = 512; p.n_seq_max = 1;
-    p.type_k = MI355_TYPE_F16; p.type_v = MI355_TYPE_F16; p.flash_attn = 1; p.embeddings = 0; p.use_graphs = 1; p.logits_to_host = 1;
+    p.type_k = MI355_TYPE_F16; p.type_v = MI355_TYPE_F16; p.flash_attn = 1; p.embeddings = 0; p.use_graphs = 1; p.logits_to_host = 1; p.exact_f32 = 0;
     return p;
 }
 
@@ -167,6 +167,7 @@ mi355_context *mi355_context_new(mi355_model *model, mi355_context_params params
     cp.embeddings = params.embeddings != 0;
     cp.use_graphs = params.use_graphs != 0;
     cp.logits_to_host = params.logits_to_host != 0;
+    cp.exact_f32 = params.exact_f32 != 0;
     if (cp.n_ctx == 0 || cp.n_batch == 0 || cp.n_seq_max > 64) { fail("bad context parameters (n_ctx and n_batch must be positive, n_seq_max at most 64)"); return nullptr; }
     MI355_GUARD(return nullptr,
         std::unique_ptr<Context> c(new Context(model->m, cp));

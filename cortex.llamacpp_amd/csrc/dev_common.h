@@ -12,15 +12,15 @@ constexpr int QK_K = 256;
 
 // ggml type ids (GGUF on-disk values)
 enum : int {
-    T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q5_0 = 6, T_Q8_0 = 8, T_Q2_K = 10, T_Q3_K = 11, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_Q8_K = 15, T_IQ4_NL = 20,
+    T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q5_0 = 6, T_Q8_0 = 8, T_Q2_K = 10, T_Q3_K = 11, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_Q8_K = 15, T_IQ4_NL = 20, T_BF16 = 30,
 };
 
 // ---- ggml on-disk block sizes ------------------------------------------------------------
 __host__ __device__ constexpr int ggml_block_elems(int t) {
-    return (t == T_F32 || t == T_F16) ? 1 : (t == T_Q4_0 || t == T_Q5_0 || t == T_Q8_0 || t == T_IQ4_NL) ? 32 : 256;
+    return (t == T_F32 || t == T_F16 || t == T_BF16) ? 1 : (t == T_Q4_0 || t == T_Q5_0 || t == T_Q8_0 || t == T_IQ4_NL) ? 32 : 256;
 }
 __host__ __device__ constexpr int ggml_block_bytes(int t) {
-    return t == T_F32 ? 4 : t == T_F16 ? 2 : t == T_Q4_0 ? 18 : t == T_Q8_0 ? 34 : t == T_Q4_K ? 144 :
+    return t == T_F32 ? 4 : (t == T_F16 || t == T_BF16) ? 2 : t == T_Q4_0 ? 18 : t == T_Q8_0 ? 34 : t == T_Q4_K ? 144 :
            t == T_Q5_K ? 176 : t == T_Q6_K ? 210 : t == T_Q8_K ? 292 : t == T_Q2_K ? 84 : t == T_Q3_K ? 110 : t == T_Q5_0 ? 22 : t == T_IQ4_NL ? 18 : 0;
 }
 __host__ __device__ inline size_t ggml_row_bytes(int t, int64_t n) {

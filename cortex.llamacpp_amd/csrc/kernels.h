@@ -256,6 +256,76 @@ hipError_t launch_moe_gather_act(const ActQuant &src, const int32_t *tok_of, int
 // x[t][d] += sum_j y[slot_of[t*k + j]][d] * w[t][j]   (same order of operations as launch_moe_combine)
 hipError_t launch_moe_scatter_combine(float *x, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, hipStream_t st);
 
+// ---------------------------------------------------------------- BF16-weight linear layers (mmb.hip)
+// Y[z][t][n] = epi(sum_k X[z][t][k] W[z][n][k]): f32 activations, bf16 weight rows (K-contiguous, stride ldw), f32 accumulation.
+// f32 = 1: every product in true 32-bit arithmetic (the weights widen exactly); 0: batches round the activations to bf16 for the matrix cores.
+// Outer index z < nz, one of: plain strides (x_zs / w_zs / y_zs elements; per-head products); meta != nullptr: z is an expert, its rows of X and Y are
+// [meta[nz + z], + meta[z]) (launch_moe_group's counts | offsets; T = upper bound of any expert's rows); sel != nullptr: z is a (token, rank) pair - weight set
+// sel[z], row z / sel_div of X, row z of Y.
+enum { MMB_STORE = 0, MMB_RELU2 = 1, MMB_SILU_MUL = 2 };       // y | relu(y)^2 | silu(W x) * (W2 x)
+constexpr int MMB_VEC_ROWS = 16;                               // up to this many rows take the one-wave-per-column kernel
+struct MMBArgs {
+    const float *x = nullptr; int ldx = 0;
+    const unsigned short *w = nullptr, *w2 = nullptr; int ldw = 0;
+    float *y = nullptr; int ldy = 0;
+    int T = 0, N = 0, K = 0, epi = MMB_STORE, f32 = 0;
+    float out_scale = 1.0f;                                    // multiplies every stored value (a model's logit scale)
+    int nz = 1; long long x_zs = 0, w_zs = 0, y_zs = 0;
+    const int32_t *meta = nullptr;
+    const int32_t *sel = nullptr; int sel_div = 1;
+};
+hipError_t launch_mmb(const MMBArgs &a, hipStream_t st);
+
+// ---------------------------------------------------------------- f32 norms / row add (act.hip), table routing (misc.hip)
+// y = [resid +] x / sqrt(mean(x^2) + eps) * (w_off + w) for T rows of n (row strides ld_x, ld_y; resid shares y's indexing and may be y)
+hipError_t launch_rmsnorm_f32(const float *x, int ld_x, const float *w, float w_off, const float *resid, float *y, int ld_y, int n, int T, float eps, hipStream_t st);
+hipError_t launch_add_row(float *x, const float *row, int n, int T, hipStream_t st);                      // x[t][:] += row
+hipError_t launch_moe_table_ids(const int32_t *table, const int32_t *tok, int T, int k, int32_t *ids, hipStream_t st);   // ids[t][j] = table[tok[t]][j]
+hipError_t launch_moe_uniform_combine(float *out, const float *y, const int32_t *slot_of, int T, int E, int k, float w, hipStream_t st);
+
+// ---------------------------------------------------------------- latent attention (latent_attn.hip)
+// cache row of a cell: [kv_rank normed latent | rot rotated shared key part] f32.  rot_freq: [rot_dims / 2] angles per position (host-made, YaRN blend
+// included), rot_mscale multiplies cos and sin; interleaved pairs over the first rot_dims entries of the rotated part.
+struct LatentPrepArgs {
+    const float *a; int ld_a;              // [T][q_rank | kv_rank | rot] down-projections
+    int T, q_rank, kv_rank, rot, rot_dims;
+    const float *wq_norm, *wkv_norm; float eps;
+    const float *rot_freq; float rot_mscale;
+    const int32_t *tok_pos, *tok_cell;
+    float *cq;                             // [T][q_rank] normed query latent
+    float *cache;                          // [n_ctx][kv_rank + rot]
+};
+hipError_t launch_latent_prep(const LatentPrepArgs &a, hipStream_t st);
+struct LatentAttnArgs {
+    const float *qa; int ld_qa;            // [T][H][kv_rank]: W_uk folded into the unrotated query part
+    const float *q; int ld_q;              // [T][H][dim + rot]: the part to rotate sits behind the first dim entries of each head
+    float *out; int ld_out;                // [T][H][kv_rank]: attended latents
+    int T, H, dim, rot, kv_rank, rot_dims;
+    const float *cache;
+    const int32_t *cell_pos; const uint64_t *cell_seq; const int32_t *tok_pos, *tok_seq; const int32_t *n_kv_dev;
+    int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
+    float scale; const float *sink;        // sink: [H] or nullptr
+    const float *rot_freq; float rot_mscale;
+};
+bool latent_attn_shape_ok(int kv_rank, int rot);
+hipError_t launch_latent_attn(const LatentAttnArgs &a, hipStream_t st);
+
+// ---------------------------------------------------------------- matrix-memory recurrence (mlstm.hip)
+struct MlstmArgs {
+    const float *p; int ld_p;              // [T][q: H*D | k: H*D | v: H*VD | g: H*VD | i: H | f: H] projections of the batch
+    float *o; int ld_o;                    // [T][H][VD] un-normed outputs
+    int H, D, VD; float gate_cap;
+    const float *i_bias, *f_bias;          // [H]
+    float *S, *n, *m;                      // state of every slot: [slot][H][D][VD], [slot][H][D], [slot][H]
+    const int32_t *seg_start, *seg_len, *seg_slot; int n_seg;   // runs of consecutive batch rows of one sequence each; no slot twice in a launch
+};
+bool mlstm_shape_ok(int D, int VD);
+hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st);
+// y[t][h][j] = o / rms(o over the head) * w[h][j] * sigmoid(p[t][off_g + h * VD + j])
+hipError_t launch_mlstm_out(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int T, int H, int VD, float eps, float *y, int ld_y,
+                            hipStream_t st);
+hipError_t launch_mlstm_state_reset(float *S, size_t n_s, float *n, size_t n_n, float *m, size_t n_m, hipStream_t st);   // S = 0, n = 0, m = 0
+
 // ---------------------------------------------------------------- attention side (attn.hip)
 // words between two merge-ticket counters / hand-over flags of the decode attention kernels (attn_decode_dev.h, attn_out.hip): one 128-byte line each
 constexpr int ATT_SYNC_STRIDE = 32;

@@ -501,6 +501,30 @@ hipError_t launch_moe_gather_act(const ActQuant &src, const int32_t *tok_of, int
     hipLaunchKernelGGL(moe_gather_act_kernel, dim3(n_rows), dim3(256), 0, st, src, tok_of, K, dst);
     return hipGetLastError();
 }
+// Routing without a router: a table [n_vocab][k] names the experts of every token id; ids[t * k + j] = table[tok[t] * k + j]
+__global__ void moe_table_ids_kernel(const int32_t *table, const int32_t *tok, int k, int n, int32_t *ids) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) ids[i] = table[(size_t)tok[i / k] * k + (i % k)];
+}
+hipError_t launch_moe_table_ids(const int32_t *table, const int32_t *tok, int T, int k, int32_t *ids, hipStream_t st) {
+    if (T * k <= 0) return hipSuccess;
+    hipLaunchKernelGGL(moe_table_ids_kernel, dim3((unsigned)((T * k + 255) / 256)), dim3(256), 0, st, table, tok, k, T * k, ids);
+    return hipGetLastError();
+}
+// out[t][d] = w * sum_j y[row(t, j)][d], experts added in rank order; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
+__global__ void moe_uniform_combine_kernel(float *out, const float *y, const int32_t *slot_of, int T, int E, int k, float w) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)T * E) return;
+    const int t = (int)(i / E), d = (int)(i - (int64_t)t * E);
+    float o = 0.0f;
+    for (int j = 0; j < k; j++) o += y[(size_t)(slot_of ? slot_of[(size_t)t * k + j] : t * k + j) * E + d];
+    out[i] = o * w;
+}
+hipError_t launch_moe_uniform_combine(float *out, const float *y, const int32_t *slot_of, int T, int E, int k, float w, hipStream_t st) {
+    if ((int64_t)T * E <= 0) return hipSuccess;
+    hipLaunchKernelGGL(moe_uniform_combine_kernel, dim3((unsigned)(((int64_t)T * E + 255) / 256)), dim3(256), 0, st, out, y, slot_of, T, E, k, w);
+    return hipGetLastError();
+}
 __global__ void moe_scatter_combine_kernel(float *x, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (int64_t)T * E) return;

@@ -1,0 +1,263 @@
+// mmb.hip — linear layers against BF16 weight rows ([out][in], K-contiguous) with f32 activations and f32 accumulation:
+//
+//   Y[z][t][n] = epi( sum_k X[z][t][k] * W[z][n][k] )
+//
+// z is an optional outer index with its own element strides on every operand: the heads of a per-head product (latent attention folds W_uk into the query
+// and unfolds the attended latent through W_uv), the experts of a grouped batch (rows [offs[z], offs[z] + counts[z]) of X and Y belong to expert z), or
+// the (token, rank) pairs of a few single tokens that picked their experts (sel[z] names the weight set, row z of Y, row z / sel_div of X).
+//
+// Three kernels behind one launch:
+//   * mmb_vec   - up to a few dozen rows: one wave per output column walks K with 16-byte weight loads, the activations stay f32.  Weight-stream bound, the
+//                 form of every single-token step in both precisions.
+//   * mmb_mfma  - batches in bf16 mode: activations rounded to bf16 in registers, v_mfma_f32_32x32x16_bf16, one 32 x 32 (or 64 x 64) tile per wave, both operands
+//                 read K-contiguous straight into the matrix-core register layout (lane = (row, k-group of 8)).
+//   * mmb_f32   - batches in f32 mode (and every shape the other two refuse): LDS-tiled, v_fma_f32 only - products of an f32 activation and a bf16 weight
+//                 widened exactly, no reduced-precision matrix mode anywhere.
+// Epilogues: store | relu(y)^2 | silu(W x) * (W2 x) (two weight sets, one pass over the activations).
+#include "kernels.h"
+
+namespace mi355 {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+__device__ __forceinline__ unsigned short f2bf(float f) {                       // round to nearest even (NaN stays NaN)
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float epi_apply(int epi, float a, float b) {
+    if (epi == MMB_RELU2) { const float r = a > 0.0f ? a : 0.0f; return r * r; }
+    if (epi == MMB_SILU_MUL) return a / (1.0f + expf(-a)) * b;
+    return a;
+}
+
+// where the rows of outer index z live: first row and row count of X / Y, the weight set
+struct ZView { const float *x; const unsigned short *w, *w2; float *y; int rows; };
+__device__ __forceinline__ ZView z_view(const MMBArgs &a, int z) {
+    ZView v;
+    int wz = z, x0 = 0, y0 = 0;
+    v.rows = a.T;
+    if (a.sel) { wz = a.sel[z]; x0 = z / a.sel_div; y0 = z; v.rows = 1; }
+    else if (a.meta) { v.rows = a.meta[z]; x0 = y0 = a.meta[a.nz + z]; }
+    v.x = a.x + (size_t)(a.sel || a.meta ? 0 : z) * a.x_zs + (size_t)x0 * a.ldx;
+    v.y = a.y + (size_t)(a.sel || a.meta ? 0 : z) * a.y_zs + (size_t)y0 * a.ldy;
+    v.w = a.w + (size_t)wz * a.w_zs;
+    v.w2 = a.w2 ? a.w2 + (size_t)wz * a.w_zs : nullptr;
+    return v;
+}
+
+// ---------------------------------------------------------------- few rows: one wave per output column
+template <bool VEC>
+__global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = blockIdx.x * 4 + wave;
+    const ZView v = z_view(a, blockIdx.y);
+    if (n >= a.N) return;
+    const unsigned short *wr = v.w + (size_t)n * a.ldw, *wr2 = v.w2 ? v.w2 + (size_t)n * a.ldw : nullptr;
+    constexpr int TB = 8;
+    for (int t0 = 0; t0 < v.rows; t0 += TB) {
+        float acc[TB], acc2[TB];
+#pragma unroll
+        for (int i = 0; i < TB; i++) { acc[i] = 0.0f; acc2[i] = 0.0f; }
+        const int nt = v.rows - t0 < TB ? v.rows - t0 : TB;
+        if (VEC) {
+            for (int k = lane * 8; k < a.K; k += 512) {
+                const u16x8 w8 = *reinterpret_cast<const u16x8 *>(wr + k);
+                u16x8 w28 = w8;
+                if (wr2) w28 = *reinterpret_cast<const u16x8 *>(wr2 + k);
+#pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    if (i >= nt) break;
+                    const float *xr = v.x + (size_t)(t0 + i) * a.ldx + k;
+                    const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr), x1 = *reinterpret_cast<const f32x4 *>(xr + 4);
+                    const float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        acc[i] = fmaf(xs[e], bf2f(w8[e]), acc[i]);
+                        if (wr2) acc2[i] = fmaf(xs[e], bf2f(w28[e]), acc2[i]);
+                    }
+                }
+            }
+        } else {
+            for (int k = lane; k < a.K; k += 64) {
+                const float w = bf2f(wr[k]), w2 = wr2 ? bf2f(wr2[k]) : 0.0f;
+#pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    if (i >= nt) break;
+                    const float x = v.x[(size_t)(t0 + i) * a.ldx + k];
+                    acc[i] = fmaf(x, w, acc[i]);
+                    acc2[i] = fmaf(x, w2, acc2[i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TB; i++) {
+            if (i >= nt) break;
+            float s = acc[i], s2 = acc2[i];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o, 64); s2 += __shfl_xor(s2, o, 64); }
+            if (lane == 0) v.y[(size_t)(t0 + i) * a.ldy + n] = epi_apply(a.epi, s, s2) * a.out_scale;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- batches, f32: 64 x 64 outputs per workgroup, 16 of k per stage, 4 x 4 per thread
+template <bool GATED>
+__global__ __launch_bounds__(256) void mmb_f32_kernel(MMBArgs a) {
+    constexpr int BM = 64, BN = 64, BK = 16, LD = 68;
+    __shared__ float sX[BK][LD], sW[BK][LD], sW2[GATED ? BK : 1][LD];
+    const ZView v = z_view(a, blockIdx.z);
+    const int t0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (t0 >= v.rows) return;                                   // (uniform: before any barrier)
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int lr = tid >> 2, lk = (tid & 3) * 4;                 // loader: row lr of both tiles, 4 consecutive k
+    float acc[4][4], acc2[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) { acc[i][j] = 0.0f; acc2[i][j] = 0.0f; }
+    const bool xrow = t0 + lr < v.rows, wrow = n0 + lr < a.N;
+    const float *xr = v.x + (size_t)(t0 + lr) * a.ldx;
+    const unsigned short *wr = v.w + (size_t)(n0 + lr) * a.ldw;
+    const unsigned short *wr2 = GATED ? v.w2 + (size_t)(n0 + lr) * a.ldw : nullptr;
+    for (int k0 = 0; k0 < a.K; k0 += BK) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int k = k0 + lk + e;
+            const bool in = k < a.K;
+            sX[lk + e][lr] = xrow && in ? xr[k] : 0.0f;
+            sW[lk + e][lr] = wrow && in ? bf2f(wr[k]) : 0.0f;
+            if (GATED) sW2[lk + e][lr] = wrow && in ? bf2f(wr2[k]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; k++) {
+            const f32x4 xv = *reinterpret_cast<const f32x4 *>(&sX[k][ty * 4]);
+            const f32x4 wv = *reinterpret_cast<const f32x4 *>(&sW[k][tx * 4]);
+            const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ws[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(xs[i], ws[j], acc[i][j]);
+            if (GATED) {
+                const f32x4 w2v = *reinterpret_cast<const f32x4 *>(&sW2[k][tx * 4]);
+                const float w2s[4] = {w2v.x, w2v.y, w2v.z, w2v.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) acc2[i][j] = fmaf(xs[i], w2s[j], acc2[i][j]);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int t = t0 + ty * 4 + i;
+        if (t >= v.rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int n = n0 + tx * 4 + j;
+            if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, acc[i][j], acc2[i][j]) * a.out_scale;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- batches, bf16 on the matrix cores: a wave owns WT x WT tiles of 32 x 32 outputs
+template <int WT, bool GATED>
+__global__ __launch_bounds__(256) void mmb_mfma_kernel(MMBArgs a) {
+    const ZView v = z_view(a, blockIdx.z);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, kg = lane >> 5;
+    const int n0 = blockIdx.x * (64 * WT) + (wave & 1) * (32 * WT), t0 = blockIdx.y * (64 * WT) + (wave >> 1) * (32 * WT);
+    if (n0 >= a.N || t0 >= v.rows) return;                      // (wave-uniform, no barriers in this kernel)
+    const unsigned short *wr[WT], *wr2[WT];
+    const float *xr[WT];
+#pragma unroll
+    for (int i = 0; i < WT; i++) {
+        const int n = n0 + 32 * i + m, t = t0 + 32 * i + m;     // rows past the end read the last row; their results are never stored
+        wr[i] = v.w + (size_t)(n < a.N ? n : a.N - 1) * a.ldw + 8 * kg;
+        wr2[i] = GATED ? v.w2 + (size_t)(n < a.N ? n : a.N - 1) * a.ldw + 8 * kg : nullptr;
+        xr[i] = v.x + (size_t)(t < v.rows ? t : v.rows - 1) * a.ldx + 8 * kg;
+    }
+    f32x16 acc[WT][WT], acc2[GATED ? WT : 1][GATED ? WT : 1];
+#pragma unroll
+    for (int i = 0; i < WT; i++)
+#pragma unroll
+        for (int j = 0; j < WT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; if (GATED) acc2[i][j][r] = 0.0f; }
+    for (int k0 = 0; k0 < a.K; k0 += 16) {
+        bf16x8 wa[WT], wb[GATED ? WT : 1], xb[WT];
+#pragma unroll
+        for (int i = 0; i < WT; i++) {
+            wa[i] = *reinterpret_cast<const bf16x8 *>(wr[i] + k0);
+            if (GATED) wb[i] = *reinterpret_cast<const bf16x8 *>(wr2[i] + k0);
+            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr[i] + k0), x1 = *reinterpret_cast<const f32x4 *>(xr[i] + k0 + 4);
+            u16x8 xb16 = {f2bf(x0.x), f2bf(x0.y), f2bf(x0.z), f2bf(x0.w), f2bf(x1.x), f2bf(x1.y), f2bf(x1.z), f2bf(x1.w)};
+            xb[i] = __builtin_bit_cast(bf16x8, xb16);
+        }
+#pragma unroll
+        for (int i = 0; i < WT; i++)
+#pragma unroll
+            for (int j = 0; j < WT; j++) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[i], xb[j], acc[i][j], 0, 0, 0);
+                if (GATED) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[i], xb[j], acc2[i][j], 0, 0, 0);
+            }
+    }
+    // register r of a lane: weight row (r & 3) + 8 (r >> 2) + 4 kg of the tile, token = lane & 31
+#pragma unroll
+    for (int i = 0; i < WT; i++)
+#pragma unroll
+        for (int j = 0; j < WT; j++) {
+            const int t = t0 + 32 * j + m;
+            if (t >= v.rows) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int n = n0 + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * kg;
+                if (n < a.N) v.y[(size_t)t * a.ldy + n] = epi_apply(a.epi, acc[i][j][r], GATED ? acc2[i][j][r] : 0.0f) * a.out_scale;
+            }
+        }
+}
+
+}  // namespace
+
+hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
+    if (a.T <= 0 || a.N <= 0 || a.nz <= 0) return hipSuccess;
+    if (a.K <= 0 || !a.x || !a.w || !a.y || (a.epi == MMB_SILU_MUL && !a.w2)) return hipErrorInvalidValue;
+    const bool gated = a.epi == MMB_SILU_MUL;
+    const auto al = [](const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
+    // 16-byte loads of both operands: every row start and every stride on a 16-byte boundary
+    const bool vec = (a.K % 8) == 0 && (a.ldw % 8) == 0 && (a.w_zs % 8) == 0 && (a.ldx % 4) == 0 && (a.x_zs % 4) == 0 && al(a.w, 16) && al(a.x, 16) &&
+                     (!a.w2 || al(a.w2, 16));
+    const int rows_max = a.sel ? 1 : a.T;                        // most rows any outer index can hold
+    if (rows_max <= MMB_VEC_ROWS || a.sel) {
+        const dim3 grid((unsigned)((a.N + 3) / 4), (unsigned)a.nz);
+        if (vec) hipLaunchKernelGGL(mmb_vec_kernel<true>, grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL(mmb_vec_kernel<false>, grid, dim3(256), 0, st, a);
+        return hipGetLastError();
+    }
+    if (!a.f32 && vec && (a.K % 16) == 0) {
+        const dim3 big((unsigned)((a.N + 127) / 128), (unsigned)((rows_max + 127) / 128), (unsigned)a.nz);
+        if (big.x * big.y * big.z >= 512 && !gated) hipLaunchKernelGGL((mmb_mfma_kernel<2, false>), big, dim3(256), 0, st, a);
+        else {
+            const dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((rows_max + 63) / 64), (unsigned)a.nz);
+            if (gated) hipLaunchKernelGGL((mmb_mfma_kernel<1, true>), grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((mmb_mfma_kernel<1, false>), grid, dim3(256), 0, st, a);
+        }
+        return hipGetLastError();
+    }
+    const dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((rows_max + 63) / 64), (unsigned)a.nz);
+    if (gated) hipLaunchKernelGGL(mmb_f32_kernel<true>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(mmb_f32_kernel<false>, grid, dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+}  // namespace mi355

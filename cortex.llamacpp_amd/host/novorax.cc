@@ -1,0 +1,579 @@
+// novorax.cc — loading a Novorax folder and running its layer stack inside Context (see novorax.h for the design, runtime.h for the context).
+//
+// The context's own machinery carries it: the cell table (find / free / sequence masks) addresses the latent-attention cache planes, the micro-batch staging
+// block brings tokens, positions, cells and sequence ids to the device, the sequence id is the slot of the recurrent state, logits / arg-max / top-k leave
+// through the usual buffers.  What is new per micro-batch is the list of segments (runs of consecutive rows of one sequence) the recurrence walks.
+#include <sys/stat.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+
+#include "json.h"
+#include "runtime.h"
+#include "safetensors.h"
+
+namespace mi355 {
+
+void set_error(const char *fmt, ...);
+
+#define NVX_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess) {                                                                    \
+            set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__);  \
+            return e_;                                                                             \
+        }                                                                                          \
+    } while (0)
+
+bool novorax_path(const std::string &path, std::string &dir) {
+    struct stat st;
+    if (stat(path.c_str(), &st) != 0) return false;
+    dir = path;
+    if (!S_ISDIR(st.st_mode)) {
+        const size_t sl = path.find_last_of('/');
+        const std::string base = sl == std::string::npos ? path : path.substr(sl + 1);
+        if (base != "config.json") return false;
+        dir = sl == std::string::npos ? "." : path.substr(0, sl);
+    }
+    return stat((dir + "/config.json").c_str(), &st) == 0 && stat((dir + "/model.safetensors").c_str(), &st) == 0;
+}
+
+namespace {
+
+struct Loader {
+    SafeTensorsFile st;
+    Model *m = nullptr;
+    std::string err;
+    uint64_t bytes = 0;
+
+    void *dev(const void *host, size_t n) {
+        if (!err.empty()) return nullptr;
+        void *p = nullptr;
+        if (hipMalloc(&p, n ? n : 16) != hipSuccess) { err = "device allocation of " + std::to_string(n) + " bytes failed"; return nullptr; }
+        m->arenas.push_back((uint8_t *)p);
+        if (n && hipMemcpy(p, host, n, hipMemcpyHostToDevice) != hipSuccess) { err = "upload failed"; return nullptr; }
+        bytes += n;
+        return p;
+    }
+    const SafeTensor *need(const std::string &name, const char *dtype, std::initializer_list<int64_t> shape) {
+        if (!err.empty()) return nullptr;
+        const SafeTensor *t = st.find(name);
+        if (!t) { err = "tensor '" + name + "' missing"; return nullptr; }
+        if (t->dtype != dtype) { err = "tensor '" + name + "' is " + t->dtype + ", expected " + dtype; return nullptr; }
+        if (t->shape.size() != shape.size() || !std::equal(shape.begin(), shape.end(), t->shape.begin())) {
+            std::string want, have;
+            for (int64_t d : shape) want += (want.empty() ? "" : ", ") + std::to_string(d);
+            for (int64_t d : t->shape) have += (have.empty() ? "" : ", ") + std::to_string(d);
+            err = "tensor '" + name + "' has shape [" + have + "], the configuration asks for [" + want + "]";
+            return nullptr;
+        }
+        return t;
+    }
+    // several [rows_i][K] bf16 tensors under each other as one device matrix
+    BfMat rows(const std::vector<std::pair<std::string, int>> &parts, int K) {
+        BfMat o;
+        std::vector<unsigned short> host;
+        for (const auto &pr : parts) {
+            const SafeTensor *t = need(pr.first, "BF16", {pr.second, K});
+            if (!t) return o;
+            const unsigned short *s = (const unsigned short *)t->data;
+            host.insert(host.end(), s, s + (size_t)pr.second * K);
+            o.N += pr.second;
+        }
+        o.K = K;
+        o.w = (unsigned short *)dev(host.data(), host.size() * 2);
+        return o;
+    }
+    float *vec(const std::string &name, int n) {
+        const SafeTensor *t = need(name, "BF16", {n});
+        if (!t) return nullptr;
+        std::vector<float> h((size_t)n);
+        const unsigned short *s = (const unsigned short *)t->data;
+        for (int i = 0; i < n; i++) { const uint32_t u = (uint32_t)s[i] << 16; memcpy(&h[(size_t)i], &u, 4); }
+        return (float *)dev(h.data(), h.size() * 4);
+    }
+};
+
+bool positive(std::string &err, const char *what, int64_t v, int64_t hi = 1 << 24) {
+    if (v >= 1 && v <= hi) return true;
+    err = std::string("configuration: ") + what + " = " + std::to_string(v) + " is out of range";
+    return false;
+}
+
+}  // namespace
+
+Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int &status) {
+    status = -102;
+    std::ifstream cf(dir + "/config.json");
+    if (!cf) { err = "cannot open " + dir + "/config.json"; status = -101; return nullptr; }
+    std::stringstream ss;
+    ss << cf.rdbuf();
+    Json cfg;
+    std::string jerr;
+    if (!Json::parse(ss.str(), cfg, &jerr) || !cfg.is_object()) { err = "config.json: " + jerr; return nullptr; }
+    if (cfg["architecture"].as_string() != "Novorax") { err = "config.json: unsupported architecture '" + cfg["architecture"].as_string() + "'"; return nullptr; }
+    std::unique_ptr<Model> m(new Model());
+    m->path = dir;
+    m->device = main_gpu;
+    if (hipSetDevice(main_gpu) != hipSuccess) { err = "hipSetDevice failed"; status = -103; return nullptr; }
+    Loader ld;
+    ld.m = m.get();
+    err = ld.st.open(dir + "/model.safetensors");
+    if (!err.empty()) { status = err.rfind("cannot", 0) == 0 ? -101 : -102; return nullptr; }
+    m->nvx.reset(new NovoraxModel());
+    NovoraxModel &M = *m->nvx;
+    const int W = (int)cfg["width"].as_int(), V = (int)cfg["vocab"].as_int();
+    if (!positive(err, "width", W) || !positive(err, "vocab", V)) return nullptr;
+    M.width = W; M.n_vocab = V;
+    M.eps = (float)cfg["norm"]["eps"].as_double(1e-5);
+    M.logit_scale = (float)cfg["logit_scale"].as_double(1.0);
+    const Json &layers = cfg["layers"];
+    if (!layers.is_array() || layers.size() == 0 || layers.size() > 1024) { err = "configuration: 'layers' must list 1 .. 1024 layers"; return nullptr; }
+    const int nl = (int)layers.size();
+
+    // the embedding table keeps the row stride launch_get_rows expects
+    {
+        const SafeTensor *t = ld.need("embed", "BF16", {V, W});
+        if (t) {
+            const size_t rb = dev_row_bytes(T_BF16, W);
+            std::vector<uint8_t> host((size_t)V * rb, 0);
+            for (int r = 0; r < V; r++) memcpy(host.data() + (size_t)r * rb, t->data + (size_t)r * W * 2, (size_t)W * 2);
+            M.embed.w = (unsigned short *)ld.dev(host.data(), host.size());
+            M.embed.N = V; M.embed.K = W;
+        }
+    }
+    M.head = ld.rows({{"head", V}}, W);
+    M.final_norm = ld.vec("final.norm", W);
+
+    M.layers.resize((size_t)nl);
+    for (int il = 0; il < nl && ld.err.empty(); il++) {
+        const Json &lc = layers.at((size_t)il), &mx = lc["mixer"];
+        NvxLayer &L = M.layers[(size_t)il];
+        const std::string p = "l" + std::to_string(il) + ".", pm = p + "mix.";
+        const std::string type = lc["type"].as_string();
+        L.norm1 = ld.vec(p + "norm1", W);
+        L.norm1b = ld.vec(p + "norm1b", W);
+        L.heads = (int)mx["heads"].as_int(); L.dim = (int)mx["dim"].as_int(); L.vdim = (int)mx["vdim"].as_int();
+        if (!positive(err, "mixer.heads", L.heads, 4096) || !positive(err, "mixer.dim", L.dim, 1 << 16) || !positive(err, "mixer.vdim", L.vdim, 1 << 16)) return nullptr;
+        const int H = L.heads;
+        if (type == "latent_attention") {
+            L.type = NVX_LATENT;
+            L.rot = (int)mx["rot_dim"].as_int(0); L.kv_rank = (int)mx["kv_rank"].as_int(); L.q_rank = (int)mx["q_rank"].as_int();
+            if (!positive(err, "mixer.kv_rank", L.kv_rank) || !positive(err, "mixer.q_rank", L.q_rank) || L.rot < 0) { if (err.empty()) err = "configuration: mixer.rot_dim is negative"; return nullptr; }
+            if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " is beyond what the attention kernel holds per lane (512)"; return nullptr; }
+            L.scale = (float)mx["scale"].as_double(1.0);
+            const Json &mask = mx["mask"];
+            L.window = mask.is_object() ? (int)mask["size"].as_int(0) : 0;
+            if (L.window < 0) L.window = 0;
+            const Json &rot = mx["rot"];
+            L.rot_dims = rot.is_object() ? (int)rot["dims"].as_int(L.rot) : 0;
+            if (L.rot_dims > L.rot || (L.rot_dims & 1) || L.rot_dims < 0) { err = "configuration: rot.dims must be even and at most rot_dim"; return nullptr; }
+            {
+                // radians per position of pair i: base^(-2i / dims), blended towards 1 / factor of itself where YaRN says the pair turns too slowly for the
+                // original context (ramp 0 below `lo`, 1 above `hi`); cos and sin carry the attention scale 0.1 ln(factor) + 1
+                const int half = L.rot_dims / 2;
+                const double base = rot["base"].as_double(10000.0);
+                std::vector<float> fr((size_t)std::max(half, 1), 0.0f);
+                const Json &scg = rot["scaling"];
+                double factor = 1.0, lo = 0.0, hi = 0.0;
+                const bool yarn = scg.is_object() && half > 0;
+                if (yarn) {
+                    factor = scg["factor"].as_double(1.0);
+                    const double orig = scg["original"].as_double(1.0), fast = scg["fast"].as_double(32.0), slow = scg["slow"].as_double(1.0);
+                    if (!(factor > 0.0) || !(orig > 0.0) || !(fast > 0.0) || !(slow > 0.0) || !(base > 1.0)) { err = "configuration: rot.scaling values must be positive"; return nullptr; }
+                    const auto corr = [&](double turns) { return L.rot_dims * std::log(orig / (2.0 * M_PI * turns)) / (2.0 * std::log(base)); };
+                    lo = std::max(std::floor(corr(fast)), 0.0);
+                    hi = std::min(std::ceil(corr(slow)), (double)(L.rot_dims - 1));
+                    L.rot_mscale = (float)(0.1 * std::log(factor) + 1.0);
+                }
+                for (int i = 0; i < half; i++) {
+                    double f = std::pow(base, -2.0 * i / L.rot_dims);
+                    if (yarn) {
+                        const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
+                        f = f / factor * ramp + f * (1.0 - ramp);
+                    }
+                    fr[(size_t)i] = (float)f;
+                }
+                L.rot_freq = (float *)ld.dev(fr.data(), fr.size() * 4);
+            }
+            const int QD = L.dim + L.rot;
+            L.down = ld.rows({{pm + "dq", L.q_rank}, {pm + "dkv", L.kv_rank + L.rot}}, W);
+            L.dq_norm = ld.vec(pm + "dq.norm", L.q_rank);
+            L.dkv_norm = ld.vec(pm + "dkv.norm", L.kv_rank);
+            L.uq = ld.rows({{pm + "uq", H * QD}}, L.q_rank);
+            L.uv = ld.rows({{pm + "uv", H * L.vdim}}, L.kv_rank);
+            L.o = ld.rows({{pm + "o", W}}, H * L.vdim);
+            if (ld.st.find(pm + "sink")) L.sink = ld.vec(pm + "sink", H);
+            if (const SafeTensor *t = ld.need(pm + "uk", "BF16", {(int64_t)H * L.dim, L.kv_rank})) {
+                const unsigned short *s = (const unsigned short *)t->data;
+                std::vector<unsigned short> tr((size_t)H * L.kv_rank * L.dim);
+                for (int h = 0; h < H; h++)
+                    for (int d = 0; d < L.dim; d++)
+                        for (int r = 0; r < L.kv_rank; r++) tr[((size_t)h * L.kv_rank + r) * L.dim + d] = s[((size_t)h * L.dim + d) * L.kv_rank + r];
+                L.uk_t.w = (unsigned short *)ld.dev(tr.data(), tr.size() * 2);
+                L.uk_t.N = L.kv_rank; L.uk_t.K = L.dim;
+            }
+            M.max_down = std::max(M.max_down, L.q_rank + L.kv_rank + L.rot);
+            M.max_q_rank = std::max(M.max_q_rank, L.q_rank);
+            M.max_q = std::max(M.max_q, H * QD);
+            M.max_qa = std::max(M.max_qa, H * L.kv_rank);
+            M.max_att = std::max(M.max_att, H * L.vdim);
+        } else if (type == "mlstm") {
+            L.type = NVX_MLSTM;
+            L.gate_cap = (float)mx["gate_cap"].as_double(0.0);
+            if (!(L.gate_cap > 0.0f)) { err = "configuration: mixer.gate_cap must be positive"; return nullptr; }
+            if (!mlstm_shape_ok(L.dim, L.vdim)) { err = "mlstm: dim " + std::to_string(L.dim) + " is beyond what the recurrence kernel keeps in registers (256)"; return nullptr; }
+            L.proj = ld.rows({{pm + "q", H * L.dim}, {pm + "k", H * L.dim}, {pm + "v", H * L.vdim}, {pm + "g", H * L.vdim}, {pm + "i", H}, {pm + "f", H}}, W);
+            L.i_bias = ld.vec(pm + "i.b", H);
+            L.f_bias = ld.vec(pm + "f.b", H);
+            L.mix_norm = ld.vec(pm + "norm", H * L.vdim);
+            L.o = ld.rows({{pm + "o", W}}, H * L.vdim);
+            M.max_proj = std::max(M.max_proj, L.proj.N);
+            M.max_att = std::max(M.max_att, H * L.vdim);
+        } else { err = "configuration: layer " + std::to_string(il) + " has unknown type '" + type + "'"; return nullptr; }
+        const Json &mlp = lc["mlp"];
+        if (mlp.is_object()) {
+            const std::string pf = p + "mlp.";
+            L.norm2 = ld.vec(p + "norm2", W);
+            L.norm2b = ld.vec(p + "norm2b", W);
+            const std::string kind = mlp["kind"].as_string();
+            if (kind == "dense") {
+                L.ff_kind = NVX_FF_DENSE;
+                L.ff = (int)mlp["ff"].as_int();
+                if (!positive(err, "mlp.ff", L.ff)) return nullptr;
+                L.up = ld.rows({{pf + "up", L.ff}}, W);
+                L.down_ff = ld.rows({{pf + "down", W}}, L.ff);
+            } else if (kind == "moe") {
+                L.ff_kind = NVX_FF_EXPERTS;
+                L.ff = (int)mlp["expert"]["ff"].as_int();
+                L.n_expert = (int)mlp["router"]["experts"].as_int(); L.top = (int)mlp["router"]["top"].as_int();
+                if (!positive(err, "mlp.expert.ff", L.ff) || !positive(err, "mlp.router.experts", L.n_expert, 4096) || !positive(err, "mlp.router.top", L.top, L.n_expert)) return nullptr;
+                std::vector<std::pair<std::string, int>> g, u, d;
+                for (int e = 0; e < L.n_expert; e++) {
+                    const std::string pe = pf + "e" + std::to_string(e) + ".";
+                    g.push_back({pe + "gate", L.ff}); u.push_back({pe + "up", L.ff}); d.push_back({pe + "down", W});
+                }
+                L.e_gate = ld.rows(g, W); L.e_up = ld.rows(u, W); L.e_down = ld.rows(d, L.ff);
+                if (const SafeTensor *t = ld.need(pf + "table", "I32", {V, L.top})) {
+                    const int32_t *tb = (const int32_t *)t->data;
+                    for (int64_t i = 0; i < (int64_t)V * L.top; i++)
+                        if (tb[i] < 0 || tb[i] >= L.n_expert) { err = "tensor '" + pf + "table' names expert " + std::to_string(tb[i]) + " of " + std::to_string(L.n_expert); return nullptr; }
+                    L.table = (int32_t *)ld.dev(t->data, t->bytes);
+                }
+                M.max_top = std::max(M.max_top, L.top);
+                M.max_expert = std::max(M.max_expert, L.n_expert);
+            } else { err = "configuration: layer " + std::to_string(il) + " has unknown mlp.kind '" + kind + "'"; return nullptr; }
+            M.max_ff = std::max(M.max_ff, L.ff);
+        }
+    }
+    if (!ld.err.empty()) { err = ld.err; return nullptr; }
+
+    // the order of layer runs: layers before the looped span once, the span `times` times (each pass opens with the input projection), the rest once
+    int a = 0, b = 0, times = 0;
+    const Json &loop = cfg["loop"];
+    if (loop.is_object()) {
+        a = (int)loop["start"].as_int(0); b = (int)loop["stop"].as_int(0); times = (int)loop["times"].as_int(1);
+        if (a < 0 || b > nl || times < 0 || times > 4096) { err = "configuration: loop start / stop / times out of range"; return nullptr; }
+        if (b <= a || times < 1) { a = b = 0; times = 0; }
+    }
+    const auto add_run = [&](int il, int pass) {
+        NvxRun r; r.layer = il; r.pass = pass;
+        r.plane = M.layers[(size_t)il].type == NVX_LATENT ? M.n_latent_runs++ : M.n_mlstm_runs++;
+        M.runs.push_back(r);
+    };
+    for (int i = 0; i < a; i++) add_run(i, -1);
+    for (int t = 0; t < times; t++) for (int i = a; i < b; i++) add_run(i, i == a ? t : -1);
+    for (int i = b; i < nl; i++) add_run(i, -1);
+    if (times > 0) {
+        M.loop_in = ld.rows({{"loop.in", W}}, 2 * W);
+        if (const SafeTensor *t = ld.need("loop.step", "BF16", {times, W})) {
+            std::vector<float> h((size_t)times * W);
+            const unsigned short *s = (const unsigned short *)t->data;
+            for (size_t i = 0; i < h.size(); i++) { const uint32_t u = (uint32_t)s[i] << 16; memcpy(&h[i], &u, 4); }
+            M.loop_step = (float *)ld.dev(h.data(), h.size() * 4);
+        }
+    }
+    if (!ld.err.empty()) { err = ld.err; return nullptr; }
+    if (hipDeviceSynchronize() != hipSuccess) { err = "device synchronise failed after the upload"; status = -103; return nullptr; }
+
+    HParams &hp = m->hp;
+    hp.arch = "novorax";
+    hp.n_embd = W; hp.n_vocab = V; hp.n_vocab_local = V; hp.n_layer = nl; hp.n_layer_runs = (int)M.runs.size();
+    hp.n_head = M.layers[0].heads; hp.n_head_kv = 1; hp.head_dim = M.layers[0].dim; hp.eps = M.eps;
+    hp.n_head_full = hp.n_head; hp.n_head_kv_full = 1;
+    m->device_bytes = ld.bytes;
+    m->file_tensor_bytes = ld.st.file_bytes();
+    m->bytes_per_token = ld.bytes;
+    m->desc = "novorax " + std::to_string(nl) + " layers (" + std::to_string(M.runs.size()) + " runs) width " + std::to_string(W) + " BF16";
+    status = 0;
+    return m.release();
+}
+
+// ------------------------------------------------------------------------------------------ context
+bool Context::init_novorax(std::string &err) {
+    const NovoraxModel &M = *model->nvx;
+    const size_t T = cp.n_ubatch, W = (size_t)M.width, NC = cp.n_ctx, NS = cp.n_seq_max;
+    cells_.assign(NC, KVCell());
+    d_cell_pos_ = (int32_t *)dalloc(NC * 4);
+    d_cell_seq_ = (uint64_t *)dalloc(NC * 8);
+    d_delta_ = (int32_t *)dalloc(NC * 4);
+    const size_t Tp = (T + 1) & ~(size_t)1;
+    stage_bytes_ = 16 + Tp * 4 * 5 + Tp * 8;
+    stage_bytes_ = (stage_bytes_ + 15) & ~(size_t)15;
+    d_stage_ = (uint8_t *)dalloc(stage_bytes_);
+    if (!d_stage_ || hipHostMalloc((void **)&h_stage_, stage_bytes_, hipHostMallocDefault) != hipSuccess) { err = "staging allocation failed"; return false; }
+    d_nkv_ = (int32_t *)d_stage_;
+    d_tok_ = (int32_t *)(d_stage_ + 16);
+    d_pos_ = d_tok_ + Tp; d_seq_ = d_pos_ + Tp; d_cell_ = d_seq_ + Tp; d_outrow_ = d_cell_ + Tp;
+    d_seqmask_ = (uint64_t *)(d_outrow_ + Tp);
+    d_seg_ = (int32_t *)dalloc(3 * T * 4);
+    if (!d_seg_ || hipHostMalloc((void **)&h_seg_, 3 * T * 4, hipHostMallocDefault) != hipSuccess) { err = "segment list allocation failed"; return false; }
+
+    // cache planes and recurrent state
+    nvx_cache_.assign((size_t)M.n_latent_runs, nullptr);
+    nvx_S_.assign((size_t)M.n_mlstm_runs, nullptr); nvx_n_ = nvx_S_; nvx_m_ = nvx_S_;
+    for (const NvxRun &r : M.runs) {
+        const NvxLayer &L = M.layers[(size_t)r.layer];
+        if (L.type == NVX_LATENT) {
+            nvx_cache_[(size_t)r.plane] = (float *)dalloc(NC * (size_t)(L.kv_rank + L.rot) * 4);
+            if (!nvx_cache_[(size_t)r.plane]) { err = "latent cache allocation failed"; return false; }
+        } else {
+            const size_t HS = (size_t)L.heads;
+            nvx_S_[(size_t)r.plane] = (float *)dalloc(NS * HS * L.dim * L.vdim * 4);
+            nvx_n_[(size_t)r.plane] = (float *)dalloc(NS * HS * L.dim * 4);
+            nvx_m_[(size_t)r.plane] = (float *)dalloc(NS * HS * 4);
+            if (!nvx_S_[(size_t)r.plane] || !nvx_n_[(size_t)r.plane] || !nvx_m_[(size_t)r.plane]) { err = "recurrent state allocation failed"; return false; }
+        }
+    }
+    nvx_seq_len_.assign(NS, 0);
+    // activations
+    const size_t A = (size_t)std::max(M.max_down, M.max_proj), TOP = (size_t)std::max(M.max_top, 1);
+    x_ = (float *)dalloc(T * W * 4);
+    xn_ = (float *)dalloc(T * W * 4);
+    xo_ = (float *)dalloc(T * W * 4);
+    nvx_x0_ = (float *)dalloc(T * W * 4);
+    nvx_xcat_ = (float *)dalloc(T * 2 * W * 4);
+    nvx_y_ = (float *)dalloc(T * W * 4);
+    nvx_a_ = (float *)dalloc(T * std::max<size_t>(A, 1) * 4);
+    nvx_cq_ = (float *)dalloc(T * (size_t)std::max(M.max_q_rank, 1) * 4);
+    nvx_q_ = (float *)dalloc(T * (size_t)std::max(M.max_q, 1) * 4);
+    nvx_qa_ = (float *)dalloc(T * (size_t)std::max(M.max_qa, 1) * 4);
+    nvx_lat_ = (float *)dalloc(T * (size_t)std::max(M.max_qa, 1) * 4);
+    nvx_att_ = (float *)dalloc(T * (size_t)std::max(M.max_att, 1) * 4);
+    nvx_o_ = (float *)dalloc(T * (size_t)std::max(M.max_att, 1) * 4);
+    nvx_ff_ = (float *)dalloc(T * TOP * (size_t)std::max(M.max_ff, 1) * 4);
+    if (!x_ || !xn_ || !xo_ || !nvx_x0_ || !nvx_xcat_ || !nvx_y_ || !nvx_a_ || !nvx_cq_ || !nvx_q_ || !nvx_qa_ || !nvx_lat_ || !nvx_att_ || !nvx_o_ || !nvx_ff_) { err = "activation buffer allocation failed"; return false; }
+    if (M.max_top > 0) {
+        nvx_xg_ = (float *)dalloc(T * TOP * W * 4);
+        nvx_yg_ = (float *)dalloc(T * TOP * W * 4);
+        nvx_ids_ = (int32_t *)dalloc(T * TOP * 4);
+        nvx_meta_ = (int32_t *)dalloc((size_t)(2 * M.max_expert + 1) * 4);
+        nvx_slot_ = (int32_t *)dalloc(T * TOP * 4);
+        nvx_tokof_ = (int32_t *)dalloc(T * TOP * 4);
+        if (!nvx_xg_ || !nvx_yg_ || !nvx_ids_ || !nvx_meta_ || !nvx_slot_ || !nvx_tokof_) { err = "expert batch buffers allocation failed"; return false; }
+    }
+    d_argmax_ = (int32_t *)dalloc(T * 4);
+    argmax_scratch_ = (float *)dalloc(T * 129 * 4);
+    if (!d_argmax_ || !argmax_scratch_ || hipHostMalloc((void **)&h_argmax_, T * 4, hipHostMallocDefault) != hipSuccess) { err = "arg-max buffers allocation failed"; return false; }
+    embeddings_enabled = false;
+    cp.use_graphs = false;                                      // the segment lists change the launch shapes from step to step
+    kv_clear();
+    nvx_state_reset(-1);
+    if (hipDeviceSynchronize() != hipSuccess) { err = "device synchronise failed"; return false; }
+    return true;
+}
+
+void Context::nvx_state_reset(int seq) {
+    const NovoraxModel &M = *model->nvx;
+    const size_t NS = cp.n_seq_max;
+    for (const NvxRun &r : M.runs) {
+        const NvxLayer &L = M.layers[(size_t)r.layer];
+        if (L.type != NVX_MLSTM) continue;
+        const size_t s_sz = (size_t)L.heads * L.dim * L.vdim, n_sz = (size_t)L.heads * L.dim, m_sz = (size_t)L.heads;
+        const size_t first = seq < 0 ? 0 : (size_t)seq, cnt = seq < 0 ? NS : 1;
+        if (first >= NS) continue;
+        (void)launch_mlstm_state_reset(nvx_S_[(size_t)r.plane] + first * s_sz, cnt * s_sz, nvx_n_[(size_t)r.plane] + first * n_sz, cnt * n_sz,
+                                       nvx_m_[(size_t)r.plane] + first * m_sz, cnt * m_sz, stream_);
+    }
+    if (seq < 0) std::fill(nvx_seq_len_.begin(), nvx_seq_len_.end(), 0);
+    else if ((size_t)seq < nvx_seq_len_.size()) nvx_seq_len_[(size_t)seq] = 0;
+}
+
+void Context::nvx_state_copy(int src, int dst) {
+    const NovoraxModel &M = *model->nvx;
+    const size_t NS = cp.n_seq_max;
+    if (src < 0 || dst < 0 || (size_t)src >= NS || (size_t)dst >= NS || src == dst) return;
+    for (const NvxRun &r : M.runs) {
+        const NvxLayer &L = M.layers[(size_t)r.layer];
+        if (L.type != NVX_MLSTM) continue;
+        const size_t s_sz = (size_t)L.heads * L.dim * L.vdim, n_sz = (size_t)L.heads * L.dim, m_sz = (size_t)L.heads;
+        (void)hipMemcpyAsync(nvx_S_[(size_t)r.plane] + dst * s_sz, nvx_S_[(size_t)r.plane] + src * s_sz, s_sz * 4, hipMemcpyDeviceToDevice, stream_);
+        (void)hipMemcpyAsync(nvx_n_[(size_t)r.plane] + dst * n_sz, nvx_n_[(size_t)r.plane] + src * n_sz, n_sz * 4, hipMemcpyDeviceToDevice, stream_);
+        (void)hipMemcpyAsync(nvx_m_[(size_t)r.plane] + dst * m_sz, nvx_m_[(size_t)r.plane] + src * m_sz, m_sz * 4, hipMemcpyDeviceToDevice, stream_);
+    }
+    nvx_seq_len_[(size_t)dst] = nvx_seq_len_[(size_t)src];
+}
+
+bool Context::nvx_stage_segments(int n, const int32_t *seq) {
+    const size_t T = cp.n_ubatch;
+    int32_t *start = h_seg_, *len = h_seg_ + T, *slot = h_seg_ + 2 * T;
+    int ns = 0;
+    for (int i = 0; i < n; i++) {
+        if (seq[i] < 0 || seq[i] >= (int)cp.n_seq_max) { last_error = "sequence id " + std::to_string(seq[i]) + " has no state slot (n_seq_max " + std::to_string(cp.n_seq_max) + ")"; return false; }
+        if (ns > 0 && slot[ns - 1] == seq[i]) len[ns - 1]++;
+        else { start[ns] = i; len[ns] = 1; slot[ns] = seq[i]; ns++; }
+    }
+    // segments of one launch must not share a slot: cut the list where a sequence comes back
+    nvx_waves_.clear();
+    int first = 0;
+    uint64_t seen = 0;
+    for (int s = 0; s < ns; s++) {
+        const uint64_t bit = 1ull << (slot[s] & 63);
+        if (seen & bit) { nvx_waves_.push_back({first, s - first}); first = s; seen = 0; }
+        seen |= bit;
+    }
+    if (ns > first) nvx_waves_.push_back({first, ns - first});
+    return hipMemcpyAsync(d_seg_, h_seg_, 3 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
+}
+
+hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale) {
+    MMBArgs a;
+    a.x = x; a.ldx = ldx; a.w = w.w; a.w2 = w2 ? w2->w : nullptr; a.ldw = w.K; a.y = y; a.ldy = ldy;
+    a.T = T; a.N = w.N; a.K = w.K; a.epi = epi; a.f32 = cp.exact_f32 ? 1 : 0; a.out_scale = out_scale;
+    return launch_mmb(a, stream_);
+}
+
+hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
+    const NovoraxModel &M = *model->nvx;
+    const int W = M.width;
+    if (L.ff_kind == NVX_FF_DENSE) {
+        NVX_TRY(nvx_linear(L.up, xn_, W, T, nvx_ff_, L.ff, MMB_RELU2));
+        NVX_TRY(nvx_linear(L.down_ff, nvx_ff_, L.ff, T, nvx_y_, W));
+        return hipSuccess;
+    }
+    const int k = L.top, NE = L.n_expert, P = T * k;
+    NVX_TRY(launch_moe_table_ids(L.table, d_tok_, T, k, nvx_ids_, stream_));
+    MMBArgs g;
+    g.w = L.e_gate.w; g.w2 = L.e_up.w; g.ldw = W; g.N = L.ff; g.K = W; g.epi = MMB_SILU_MUL; g.f32 = cp.exact_f32 ? 1 : 0; g.w_zs = (long long)L.ff * W;
+    g.y = nvx_ff_; g.ldy = L.ff;
+    MMBArgs d;
+    d.w = L.e_down.w; d.ldw = L.ff; d.N = W; d.K = L.ff; d.f32 = g.f32; d.w_zs = (long long)W * L.ff;
+    d.x = nvx_ff_; d.ldx = L.ff; d.y = nvx_yg_; d.ldy = W;
+    const bool grouped = P > 32 && NE <= 64 && (size_t)P * 4 <= 60 * 1024;
+    if (grouped) {
+        // every expert sees its (token, rank) pairs as one batch of rows: counting sort by expert, gather, two grouped products, combine per token
+        NVX_TRY(launch_moe_group(nvx_ids_, T, k, NE, nvx_meta_, nvx_slot_, nvx_tokof_, stream_));
+        NVX_TRY(launch_gather_rows_f32(xn_, nvx_tokof_, P, W, nvx_xg_, stream_));
+        g.x = nvx_xg_; g.ldx = W; g.T = P; g.nz = NE; g.meta = nvx_meta_;
+        d.T = P; d.nz = NE; d.meta = nvx_meta_;
+        NVX_TRY(launch_mmb(g, stream_));
+        NVX_TRY(launch_mmb(d, stream_));
+        NVX_TRY(launch_moe_uniform_combine(nvx_y_, nvx_yg_, nvx_slot_, T, W, k, 1.0f / (float)k, stream_));
+    } else {
+        // a few tokens: one product per (token, rank) pair against the weights the pair picked
+        g.x = xn_; g.ldx = W; g.T = 1; g.nz = P; g.sel = nvx_ids_; g.sel_div = k;
+        d.T = 1; d.nz = P; d.sel = nvx_ids_; d.sel_div = 1;
+        NVX_TRY(launch_mmb(g, stream_));
+        NVX_TRY(launch_mmb(d, stream_));
+        NVX_TRY(launch_moe_uniform_combine(nvx_y_, nvx_yg_, nullptr, T, W, k, 1.0f / (float)k, stream_));
+    }
+    return hipSuccess;
+}
+
+hipError_t Context::run_layers_novorax(int T) {
+    const NovoraxModel &M = *model->nvx;
+    const int W = M.width;
+    const float eps = M.eps;
+    cur_T_ = T;
+    NVX_TRY(launch_kv_meta_set(d_cell_pos_, d_cell_seq_, d_cell_, d_pos_, d_seqmask_, T, stream_));
+    NVX_TRY(launch_get_rows(T_BF16, (const uint8_t *)M.embed.w, W, d_tok_, T, x_, stream_));
+    if (M.loop_in.w) NVX_TRY(hipMemcpy2DAsync(nvx_xcat_ + W, (size_t)2 * W * 4, x_, (size_t)W * 4, (size_t)W * 4, (size_t)T, hipMemcpyDeviceToDevice, stream_));
+    prof_mark("embed");
+    int ir = 0;
+    for (const NvxRun &r : M.runs) {
+        const NvxLayer &L = M.layers[(size_t)r.layer];
+        if (r.pass >= 0) {
+            // x <- W_in [x ; x0] + step[pass]: the stream and the embedding output side by side, then the pass's own vector
+            NVX_TRY(hipMemcpy2DAsync(nvx_xcat_, (size_t)2 * W * 4, x_, (size_t)W * 4, (size_t)W * 4, (size_t)T, hipMemcpyDeviceToDevice, stream_));
+            NVX_TRY(nvx_linear(M.loop_in, nvx_xcat_, 2 * W, T, x_, W));
+            NVX_TRY(launch_add_row(x_, M.loop_step + (size_t)r.pass * W, W, T, stream_));
+        }
+        NVX_TRY(launch_rmsnorm_f32(x_, W, L.norm1, 1.0f, nullptr, xn_, W, W, T, eps, stream_));
+        const int H = L.heads;
+        if (L.type == NVX_LATENT) {
+            const int QD = L.dim + L.rot, KR = L.kv_rank, LD_A = L.q_rank + KR + L.rot;
+            float *cache = nvx_cache_[(size_t)r.plane];
+            NVX_TRY(nvx_linear(L.down, xn_, W, T, nvx_a_, LD_A));
+            LatentPrepArgs pa{};
+            pa.a = nvx_a_; pa.ld_a = LD_A; pa.T = T; pa.q_rank = L.q_rank; pa.kv_rank = KR; pa.rot = L.rot; pa.rot_dims = L.rot_dims;
+            pa.wq_norm = L.dq_norm; pa.wkv_norm = L.dkv_norm; pa.eps = eps; pa.rot_freq = L.rot_freq; pa.rot_mscale = L.rot_mscale;
+            pa.tok_pos = d_pos_; pa.tok_cell = d_cell_; pa.cq = nvx_cq_; pa.cache = cache;
+            NVX_TRY(launch_latent_prep(pa, stream_));
+            NVX_TRY(nvx_linear(L.uq, nvx_cq_, L.q_rank, T, nvx_q_, H * QD));
+            MMBArgs fa;                                         // qa[t][h] = W_uk_h^T q[t][h][:dim]
+            fa.x = nvx_q_; fa.ldx = H * QD; fa.x_zs = QD; fa.w = L.uk_t.w; fa.ldw = L.dim; fa.w_zs = (long long)KR * L.dim;
+            fa.y = nvx_qa_; fa.ldy = H * KR; fa.y_zs = KR; fa.T = T; fa.N = KR; fa.K = L.dim; fa.nz = H; fa.f32 = cp.exact_f32 ? 1 : 0;
+            NVX_TRY(launch_mmb(fa, stream_));
+            LatentAttnArgs aa{};
+            aa.qa = nvx_qa_; aa.ld_qa = H * KR; aa.q = nvx_q_; aa.ld_q = H * QD; aa.out = nvx_lat_; aa.ld_out = H * KR;
+            aa.T = T; aa.H = H; aa.dim = L.dim; aa.rot = L.rot; aa.kv_rank = KR; aa.rot_dims = L.rot_dims; aa.cache = cache;
+            aa.cell_pos = d_cell_pos_; aa.cell_seq = d_cell_seq_; aa.tok_pos = d_pos_; aa.tok_seq = d_seq_; aa.n_kv_dev = d_nkv_;
+            aa.window = L.window; aa.scale = L.scale; aa.sink = L.sink; aa.rot_freq = L.rot_freq; aa.rot_mscale = L.rot_mscale;
+            NVX_TRY(launch_latent_attn(aa, stream_));
+            MMBArgs ua;                                         // att[t][h] = W_uv_h lat[t][h]
+            ua.x = nvx_lat_; ua.ldx = H * KR; ua.x_zs = KR; ua.w = L.uv.w; ua.ldw = KR; ua.w_zs = (long long)L.vdim * KR;
+            ua.y = nvx_att_; ua.ldy = H * L.vdim; ua.y_zs = L.vdim; ua.T = T; ua.N = L.vdim; ua.K = KR; ua.nz = H; ua.f32 = fa.f32;
+            NVX_TRY(launch_mmb(ua, stream_));
+            NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
+            prof_mark("latent_attention");
+        } else {
+            const int LD_P = L.proj.N;
+            NVX_TRY(nvx_linear(L.proj, xn_, W, T, nvx_a_, LD_P));
+            MlstmArgs ma{};
+            ma.p = nvx_a_; ma.ld_p = LD_P; ma.o = nvx_o_; ma.ld_o = H * L.vdim; ma.H = H; ma.D = L.dim; ma.VD = L.vdim; ma.gate_cap = L.gate_cap;
+            ma.i_bias = L.i_bias; ma.f_bias = L.f_bias; ma.S = nvx_S_[(size_t)r.plane]; ma.n = nvx_n_[(size_t)r.plane]; ma.m = nvx_m_[(size_t)r.plane];
+            const size_t TU = cp.n_ubatch;
+            for (const auto &wv : nvx_waves_) {
+                ma.seg_start = d_seg_ + wv.first; ma.seg_len = d_seg_ + TU + wv.first; ma.seg_slot = d_seg_ + 2 * TU + wv.first; ma.n_seg = wv.second;
+                NVX_TRY(launch_mlstm_scan(ma, stream_));
+            }
+            NVX_TRY(launch_mlstm_out(nvx_o_, H * L.vdim, nvx_a_, LD_P, 2 * H * L.dim + H * L.vdim, L.mix_norm, T, H, L.vdim, eps, nvx_att_, H * L.vdim, stream_));
+            NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
+            prof_mark("mlstm");
+        }
+        NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));
+        if (L.ff_kind != NVX_FF_NONE) {
+            NVX_TRY(launch_rmsnorm_f32(x_, W, L.norm2, 1.0f, nullptr, xn_, W, W, T, eps, stream_));
+            NVX_TRY(nvx_feed_forward(L, T));
+            NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm2b, 1.0f, x_, x_, W, W, T, eps, stream_));
+            prof_mark("feed_forward");
+        }
+        if (debug_taps_ && dbg_) NVX_TRY(hipMemcpyAsync(dbg_ + (size_t)ir * cp.n_ubatch * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, stream_));
+        ir++;
+    }
+    return hipSuccess;
+}
+
+hipError_t Context::run_output_novorax(int n_out, int out_base) {
+    logits_on_host_ = false;
+    if (n_out <= 0) return hipSuccess;
+    const NovoraxModel &M = *model->nvx;
+    const int W = M.width, V = M.n_vocab;
+    float *const xo = cur_T_ == 1 && n_out == 1 ? x_ : xo_;
+    if (xo != x_) NVX_TRY(launch_gather_rows_f32(x_, d_outrow_, n_out, W, xo_, stream_));
+    NVX_TRY(launch_rmsnorm_f32(xo, W, M.final_norm, 1.0f, nullptr, xn_, W, W, n_out, M.eps, stream_));
+    float *lg = d_logits_ + (size_t)out_base * V;
+    NVX_TRY(nvx_linear(M.head, xn_, W, n_out, lg, V, MMB_STORE, nullptr, M.logit_scale));
+    prof_mark("lm_head");
+    for (int r0 = 0; r0 < n_out; r0 += (int)cp.n_ubatch) {
+        const int nr = std::min((int)cp.n_ubatch, n_out - r0);
+        NVX_TRY(launch_argmax_rows(lg + (size_t)r0 * V, V, nr, h_argmax_ + out_base + r0, argmax_scratch_, (int)cp.n_ubatch, stream_));
+    }
+    prof_mark("argmax");
+    return hipSuccess;
+}
+
+}  // namespace mi355

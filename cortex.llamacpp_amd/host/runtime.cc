@@ -57,6 +57,13 @@ static bool type_supported(int t) {
 
 Model *model_load(const std::string &path, int main_gpu, std::string &err, int &status, int prefill_planes, int tp_rank, int tp_size) {
     status = 0;
+    {
+        std::string dir;                                        // a folder with config.json + model.safetensors: the Novorax loader (novorax.cc)
+        if (novorax_path(path, dir)) {
+            if (tp_size > 1) { err = "row split of a Novorax model is not supported"; status = -102; return nullptr; }
+            return novorax_load(dir, main_gpu, err, status);
+        }
+    }
     std::unique_ptr<Model> m(new Model());
     m->file.reset(new GGUFFile());
     m->path = path;
@@ -535,6 +542,7 @@ Context::~Context() {
     if (h_argmax_) (void)hipHostFree(h_argmax_);
     if (h_embd_) (void)hipHostFree(h_embd_);
     if (h_chunks_) (void)hipHostFree(h_chunks_);
+    if (h_seg_) (void)hipHostFree(h_seg_);
     if (h_mega_flag_) (void)hipHostFree(h_mega_flag_);
     if (h_topk_) (void)hipHostFree(h_topk_);
     if (h_topk_adj_) (void)hipHostFree(h_topk_adj_);
@@ -590,6 +598,7 @@ bool Context::init(std::string &err) {
     err_epoch_seen_ = stream_error_epoch();
     if (unsigned *ew = stream_error_word()) { mmvq_stream_set_error_word(ew); decode_engine_set_error_word(ew); attn_out_set_error_word(ew); tp_p2p_set_error_word(ew); }   // (per device: the pointer lives in device globals)
 
+    if (model->nvx) return init_novorax(err);
     const size_t T = cp.n_ubatch, E = hp.n_embd, FF = hp.n_ff, G = hp.n_head_kv, D = hp.head_dim, NC = cp.n_ctx;
     cells_.assign(NC, KVCell());
     kv_.resize((size_t)hp.n_layer);
@@ -720,6 +729,7 @@ bool Context::init(std::string &err) {
 
 // ------------------------------------------------------------------------------------------ KV cells
 void Context::kv_clear() {
+    if (model->nvx && stream_) nvx_state_reset(-1);
     for (auto &c : cells_) c = KVCell();
     head_ = 0;
     has_shift_ = false;
@@ -730,6 +740,14 @@ bool Context::kv_seq_rm(int seq, int p0, int p1) {
     if (seq >= 64) return false;                                   // (the cell masks are 64 bits wide)
     if (p0 < 0) p0 = 0;
     if (p1 < 0) p1 = 0x7fffffff;
+    if (model->nvx && model->nvx->n_mlstm_runs > 0) {
+        // a recurrent state cannot be cut back to an earlier position: a sequence goes as a whole (its state slot starts over), or not at all
+        for (int sq = 0; sq < (int)nvx_seq_len_.size(); sq++) {
+            if (seq >= 0 && sq != seq) continue;
+            if (p0 > 0 && (uint64_t)p0 < nvx_seq_len_[(size_t)sq]) return false;
+            if (p0 == 0) nvx_state_reset(sq);
+        }
+    }
     int new_head = (int)cells_.size();
     for (int i = 0; i < (int)cells_.size(); i++) {
         KVCell &c = cells_[(size_t)i];
@@ -748,12 +766,14 @@ void Context::kv_seq_cp(int src, int dst, int p0, int p1) {
     if (src == dst || src < 0 || dst < 0 || src >= 64 || dst >= 64) return;
     if (p0 < 0) p0 = 0;
     if (p1 < 0) p1 = 0x7fffffff;
+    if (model->nvx && p0 == 0) nvx_state_copy(src, dst);             // the recurrent state goes with a copy of the whole sequence
     for (auto &c : cells_)
         if ((c.seqs & (1ull << src)) && c.pos >= p0 && c.pos < p1) c.seqs |= 1ull << dst;
     meta_dirty_ = true;
 }
 void Context::kv_seq_add(int seq, int p0, int p1, int delta) {
     if (seq < 0 || seq >= 64) return;
+    if (model->nvx) return;                                          // positions of a Novorax sequence cannot be shifted (the state has absorbed them)
     if (p0 < 0) p0 = 0;
     if (p1 < 0) p1 = 0x7fffffff;
     if (p0 == p1 || delta == 0) return;
@@ -1885,7 +1905,7 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
         }
     }
     bool lists_usable = false;                                 // only the split-per-chunk attention kernels walk the lists
-    {
+    if (!model->nvx) {
         const HParams &hp = model->hp;
         RopeArgs ra = rope_args(*model, false);
         AttnArgs aa{};
@@ -1913,10 +1933,26 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
     // the previous step's token / position block); MI355_PROFILER_SAFE=1 drains the stream around the transfers
     static const bool profiler_safe = getenv("MI355_PROFILER_SAFE") && getenv("MI355_PROFILER_SAFE")[0] == '1';
     if (profiler_safe) (void)hipStreamSynchronize(stream_);
+    if (model->nvx) {
+        if (!nvx_stage_segments(n, seq)) { if (last_error.empty()) last_error = "segment list upload failed"; return -1; }
+        for (int i = 0; i < n; i++) nvx_seq_len_[(size_t)seq[i]] = std::max<uint64_t>(nvx_seq_len_[(size_t)seq[i]], (uint64_t)pos[i] + 1);
+    }
     if (!stage_event_) (void)hipEventCreateWithFlags(&stage_event_, hipEventDisableTiming);
     if (stage_event_) (void)hipEventRecord(stage_event_, stream_);
 
     const int V = model->hp.n_vocab;
+    if (model->nvx) {
+        if (ub_embd_) { last_error = "a Novorax model takes token ids, not embeddings"; return -1; }
+        prof_begin();
+        hipError_t en = run_layers_novorax(n);
+        if (en == hipSuccess) en = run_output_novorax(n_out, out_base);
+        if (en == hipSuccess && n_out > 0 && cp.logits_to_host)
+            en = hipMemcpyAsync(h_logits_ + (size_t)out_base * V, d_logits_ + (size_t)out_base * V, (size_t)n_out * V * 4, hipMemcpyDeviceToHost, stream_);
+        prof_end();
+        if (en != hipSuccess) { last_error = std::string("decode failed: ") + hipGetErrorString(en) + " / " + last_error_string(); return -1; }
+        dbg_tokens_ = n;
+        return 0;
+    }
     if (n == 1 && !model->hp.encoder && !ub_embd_) { (void)mega_prepare(); (void)engine_prepare(); }   // allocate and upload on first use: must not happen inside a stream capture
     // a single-token step would launch the attention + attn_output kernel whose workgroups wait for each other: only while no other context of this device has
     // such a step in flight (runtime.h fused_acquire); otherwise this step takes the wait-free launches, eagerly (the captured graphs hold the fused kernel)
@@ -2035,7 +2071,7 @@ int Context::decode(int n_tokens, const int32_t *tokens, const int32_t *pos, con
     // bidirectional attention: every token of a sequence must see all the others, so a batch is never cut into micro-batches (llama.cpp asks the same: n_ubatch >= n_tokens)
     if (hp.encoder && (size_t)n_tokens > cp.n_ubatch) { last_error = "encoder model: a batch of " + std::to_string(n_tokens) + " tokens does not fit one micro-batch (n_ubatch " + std::to_string(cp.n_ubatch) + ")"; return -1; }
     if (has_shift_) apply_k_shift();
-    if (debug_taps_ && !dbg_) dbg_ = (float *)dalloc((size_t)hp.n_layer * cp.n_ubatch * hp.n_embd * 4);
+    if (debug_taps_ && !dbg_) dbg_ = (float *)dalloc((size_t)std::max(hp.n_layer, hp.n_layer_runs) * cp.n_ubatch * hp.n_embd * 4);
 
     std::vector<int32_t> seq((size_t)n_tokens);
     std::vector<uint64_t> mask((size_t)n_tokens);
@@ -2228,7 +2264,7 @@ int Context::topk_ith(int i, int k, const TopkAdj &adj, int32_t *toks, float *lo
 
 int Context::debug_layer_out(int il, float *dst, size_t cap) {
     const HParams &hp = model->hp;
-    if (!dbg_ || il < 0 || il >= hp.n_layer) return -1;
+    if (!dbg_ || il < 0 || il >= std::max(hp.n_layer, hp.n_layer_runs)) return -1;
     const size_t n = (size_t)dbg_tokens_ * hp.n_embd;
     if (cap < n) return -1;
     (void)hipStreamSynchronize(stream_);

@@ -15,6 +15,7 @@
 
 #include "../csrc/kernels.h"
 #include "gguf.h"
+#include "novorax.h"
 
 namespace mi355 {
 
@@ -61,6 +62,7 @@ struct HParams {
     bool tp_exchange = false;    // the process has a matching group: partial sums and logits slices go through it
     int n_head_full = 0, n_head_kv_full = 0, n_ff_full = 0;
     int n_vocab_local = 0;       // rows of the output projection held here (n_vocab when it is not split)
+    int n_layer_runs = 0;        // layer executions of one forward pass (n_layer unless a span of layers runs several times; debug taps are per run)
 };
 
 struct Model {
@@ -72,6 +74,7 @@ struct Model {
     DevTensor tok_embd, out_norm, output, rope_freqs;
     DevTensor tok_types, tok_norm, tok_norm_b;       // encoder files: token-type table (row 0 is added to every token), LayerNorm of the embeddings
     std::vector<LayerWeights> layers;
+    std::unique_ptr<NovoraxModel> nvx;  // architecture "Novorax" (a folder with config.json + model.safetensors): its own layer stack, see novorax.h
     uint64_t device_bytes = 0, host_bytes = 0, file_tensor_bytes = 0, bytes_per_token = 0, planes_bytes = 0;
     ~Model();
 };
@@ -79,6 +82,9 @@ struct Model {
 // prefill_planes: 0 = never, 1 = always (fails when memory is short), -1 = when device memory allows (default)
 // tp_size > 1: load rank tp_rank's slice of every projection (rows of attn_q/k/v, ffn_gate/up and output; the matching
 // super-block columns of attn_output and ffn_down), cut on head and 256-element boundaries
+// a folder (or its config.json) whose "architecture" is Novorax: weights to the device, layer runs laid out (novorax.cc)
+Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int &status);
+bool novorax_path(const std::string &path, std::string &dir);   // does `path` name such a folder
 Model *model_load(const std::string &path, int main_gpu, std::string &err, int &status, int prefill_planes = -1, int tp_rank = 0, int tp_size = 1);
 
 struct KVCell {
@@ -93,6 +99,7 @@ struct ContextParams {
     int type_k = T_F16, type_v = T_F16;
     bool flash_attn = true, embeddings = false, use_graphs = true;
     bool logits_to_host = true;   // llama_decode contract: flagged logits rows are copied to host memory by the decode itself
+    bool exact_f32 = false;       // bf16-weight models: every product in true 32-bit arithmetic (default: batches round activations to bf16 for the matrix cores)
 };
 
 struct ProfileEntry { std::string name; float us; };
@@ -169,6 +176,23 @@ class Context {
     void apply_k_shift();
     hipError_t run_layers(int T, int n_kv_cap);
     hipError_t run_layers_encoder(int T, int n_kv_cap);
+    // ---- Novorax (novorax.cc): cache planes of the latent-attention runs share the cell table; the mlstm runs keep one state set per sequence id
+    bool init_novorax(std::string &err);
+    hipError_t run_layers_novorax(int T);
+    hipError_t run_output_novorax(int n_out, int out_base);
+    hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f);
+    hipError_t nvx_feed_forward(const NvxLayer &L, int T);
+    bool nvx_stage_segments(int n, const int32_t *seq);     // runs of consecutive tokens of one sequence -> segment arrays (pinned, then device)
+    void nvx_state_reset(int seq);                          // seq < 0: every slot
+    void nvx_state_copy(int src, int dst);
+    std::vector<float *> nvx_cache_;                        // [latent run] [n_ctx][kv_rank + rot]
+    std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [mlstm run] [n_seq_max][H][D][VD], [..][H][D], [..][H]
+    std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
+    float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
+    float *nvx_att_ = nullptr, *nvx_o_ = nullptr, *nvx_ff_ = nullptr, *nvx_xg_ = nullptr, *nvx_yg_ = nullptr;
+    int32_t *nvx_ids_ = nullptr, *nvx_meta_ = nullptr, *nvx_slot_ = nullptr, *nvx_tokof_ = nullptr;
+    int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [3][n_ubatch]: start, length, slot of every segment
+    std::vector<std::pair<int, int>> nvx_waves_;            // segment ranges [first, count) that may share a launch (no slot twice)
     hipError_t run_output(int n_out, int out_base);
     hipError_t linear(const DevTensor &w, const ActQuant &aq, const float *x_f32, int K, int T, float *out, int ld_out,
                       const float *resid, int epi);

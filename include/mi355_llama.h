@@ -75,6 +75,7 @@ typedef struct mi355_model_params {
 
 MI355_API mi355_model_params mi355_model_default_params(void);
 /* common_init_from_params -> llama_model_load_from_file (llama_server_context.cc:207) */
+/* path: a GGUF file, or a folder holding config.json + model.safetensors (architecture "Novorax") */
 MI355_API mi355_model *mi355_model_load_from_file(const char *path_gguf, mi355_model_params params);
 MI355_API void         mi355_model_free(mi355_model *model);
 
@@ -108,6 +109,8 @@ typedef struct mi355_context_params {
     int32_t  use_graphs;   /* capture the single-token decode step in a hipGraph (default 1) */
     int32_t  logits_to_host; /* 1 (default): flagged logits rows are copied to host by mi355_decode itself, as llama_decode
                               * does; 0: rows stay on the device until mi355_get_logits_ith asks (device-side greedy) */
+    int32_t  exact_f32;    /* models with bf16 weights: 1 = every product in true 32-bit arithmetic; 0 (default) = the serving precision
+                              * (batches round activations to bf16 for the matrix cores; norms, scores, states stay f32).  Ignored by GGUF models */
 } mi355_context_params;
 
 MI355_API mi355_context_params mi355_context_default_params(void);
