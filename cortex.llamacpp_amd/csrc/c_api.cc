@@ -139,6 +139,7 @@ uint64_t mi355_model_planes_bytes(const mi355_model *m) { return m->m->planes_by
 const char *mi355_model_desc(const mi355_model *m) { return m->m->desc.c_str(); }
 int mi355_model_meta_str(const mi355_model *m, const char *key, char *buf, size_t buf_size) {
     if (!m || !key || !buf || !buf_size) return 0;
+    if (!m->m->file) return 0;                                     // (a safetensors folder carries no key / value metadata)
     const GGUFValue *v = m->m->file->find(key);
     if (!v || v->type == GV_ARR) return 0;
     std::string s;
@@ -933,7 +934,8 @@ static Vocab *model_vocab(mi355_model *m) {
     if (!m->vocab_tried) {
         m->vocab_tried = true;
         std::string err;
-        m->vocab_ok = m->vocab.load(*m->m->file, err);
+        if (m->m->nvx) { m->vocab.init_numeric(m->m->hp.n_vocab); m->vocab_ok = true; }
+        else m->vocab_ok = m->vocab.load(*m->m->file, err);
         if (!m->vocab_ok) fail("tokenizer: " + err);
     }
     return m->vocab_ok ? &m->vocab : nullptr;

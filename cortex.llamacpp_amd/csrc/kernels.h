@@ -273,6 +273,8 @@ struct MMBArgs {
     int nz = 1; long long x_zs = 0, w_zs = 0, y_zs = 0;
     const int32_t *meta = nullptr;
     const int32_t *sel = nullptr; int sel_div = 1;
+    // prologue of the few-rows kernel (T <= MMB_VEC_ROWS): the rows of X are RMS-normed on the fly, x / sqrt(mean(x^2) + pn_eps) * (pn_off + pn_w[k])
+    const float *pn_w = nullptr; float pn_off = 0.0f, pn_eps = 0.0f;
 };
 hipError_t launch_mmb(const MMBArgs &a, hipStream_t st);
 

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(LatentPrepArgs a) {
     }
 }
 
-constexpr int LA_MAX_ACC = 8;                                   // latent values per lane: kv_rank <= 512
+constexpr int LA_MAX_ACC = 16;                                  // latent values per lane: kv_rank <= 1024
 
 // one workgroup per (token, head); its four waves take every fourth cell of the scanned range and keep their own running maximum, sum and weighted latent,
 // merged at the end together with the sink term

@@ -68,17 +68,36 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
 #pragma unroll
         for (int i = 0; i < TB; i++) { acc[i] = 0.0f; acc2[i] = 0.0f; }
         const int nt = v.rows - t0 < TB ? v.rows - t0 : TB;
+        float inv[TB];                                          // fused RMS norm of the rows: 1 / sqrt(mean(x^2) + eps), every wave for itself
+#pragma unroll
+        for (int i = 0; i < TB; i++) {
+            inv[i] = 1.0f;
+            if (a.pn_w && i < nt) {
+                float ss = 0.0f;
+                for (int k = lane; k < a.K; k += 64) { const float x = v.x[(size_t)(t0 + i) * a.ldx + k]; ss = fmaf(x, x, ss); }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+                inv[i] = 1.0f / sqrtf(ss / (float)a.K + a.pn_eps);
+            }
+        }
         if (VEC) {
             for (int k = lane * 8; k < a.K; k += 512) {
                 const u16x8 w8 = *reinterpret_cast<const u16x8 *>(wr + k);
                 u16x8 w28 = w8;
                 if (wr2) w28 = *reinterpret_cast<const u16x8 *>(wr2 + k);
+                float pw[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) pw[e] = a.pn_w ? a.pn_off + a.pn_w[k + e] : 1.0f;
 #pragma unroll
                 for (int i = 0; i < TB; i++) {
                     if (i >= nt) break;
                     const float *xr = v.x + (size_t)(t0 + i) * a.ldx + k;
                     const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr), x1 = *reinterpret_cast<const f32x4 *>(xr + 4);
-                    const float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                    float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                    if (a.pn_w) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) xs[e] = xs[e] * inv[i] * pw[e];
+                    }
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
                         acc[i] = fmaf(xs[e], bf2f(w8[e]), acc[i]);
@@ -92,7 +111,8 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
 #pragma unroll
                 for (int i = 0; i < TB; i++) {
                     if (i >= nt) break;
-                    const float x = v.x[(size_t)(t0 + i) * a.ldx + k];
+                    float x = v.x[(size_t)(t0 + i) * a.ldx + k];
+                    if (a.pn_w) x = x * inv[i] * (a.pn_off + a.pn_w[k]);
                     acc[i] = fmaf(x, w, acc[i]);
                     acc2[i] = fmaf(x, w2, acc2[i]);
                 }
@@ -238,6 +258,7 @@ hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     const bool vec = (a.K % 8) == 0 && (a.ldw % 8) == 0 && (a.w_zs % 8) == 0 && (a.ldx % 4) == 0 && (a.x_zs % 4) == 0 && al(a.w, 16) && al(a.x, 16) &&
                      (!a.w2 || al(a.w2, 16));
     const int rows_max = a.sel ? 1 : a.T;                        // most rows any outer index can hold
+    if (a.pn_w && rows_max > MMB_VEC_ROWS) return hipErrorInvalidValue;   // (the norm prologue lives in the few-rows kernel only)
     if (rows_max <= MMB_VEC_ROWS || a.sel) {
         const dim3 grid((unsigned)((a.N + 3) / 4), (unsigned)a.nz);
         if (vec) hipLaunchKernelGGL(mmb_vec_kernel<true>, grid, dim3(256), 0, st, a);

@@ -224,7 +224,7 @@ bool LlamaEngine::LoadModelImpl(const Json &body, std::string &err) {   // :547-
 
 void LlamaEngine::WarmUpModel(ServerInfo &si) {   // :1247-1267
     Json d = Json::object();
-    d["prompt"] = "Hello"; d["n_predict"] = 2; d["n_probs"] = 0;
+    d["prompt"] = si.backend->vocab().model() == "numeric" ? "0" : "Hello"; d["n_predict"] = 2; d["n_probs"] = 0;   // (a tokenizer-less model reads decimal token ids)
     const int id = si.ctx->RequestCompletion(d, false, false, -1);
     (void)si.ctx->NextResult(id);
 }

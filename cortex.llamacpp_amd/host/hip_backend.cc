@@ -189,7 +189,8 @@ std::unique_ptr<IBackend> make_hip_backend(const Json &body, BackendInfo &info, 
 
     Vocab vocab;
     std::string verr;
-    if (!vocab.load(*model->file, verr)) { err = "tokenizer: " + verr; return nullptr; }
+    if (model->nvx) vocab.init_numeric(model->hp.n_vocab);      // no tokenizer in the folder: decimal token ids are the text
+    else if (!vocab.load(*model->file, verr)) { err = "tokenizer: " + verr; return nullptr; }
     if (vocab.n_tokens() != model->hp.n_vocab) { err = "tokenizer size does not match the embedding table"; return nullptr; }
 
     ContextParams cp;
@@ -227,6 +228,7 @@ std::unique_ptr<IBackend> make_hip_backend(const Json &body, BackendInfo &info, 
     // a flagged row is not copied to the host with every step: plain greedy takes the device arg-max, the usual chains take the device top-k
     // (Sampler::plan_front), and a chain that needs the whole row (mirostat, top_k off, long penalty windows) fetches it on demand
     cp.logits_to_host = body.value<bool>("logits_to_host", false);
+    cp.exact_f32 = body.value<bool>("exact_f32", false);     // bf16-weight models: true 32-bit products (runtime.h)
     std::unique_ptr<Context> ctx(new Context(model.get(), cp));
     if (!ctx->init(err)) return nullptr;
 

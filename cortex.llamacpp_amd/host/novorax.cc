@@ -163,7 +163,7 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
             L.type = NVX_LATENT;
             L.rot = (int)mx["rot_dim"].as_int(0); L.kv_rank = (int)mx["kv_rank"].as_int(); L.q_rank = (int)mx["q_rank"].as_int();
             if (!positive(err, "mixer.kv_rank", L.kv_rank) || !positive(err, "mixer.q_rank", L.q_rank) || L.rot < 0) { if (err.empty()) err = "configuration: mixer.rot_dim is negative"; return nullptr; }
-            if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " is beyond what the attention kernel holds per lane (512)"; return nullptr; }
+            if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " is beyond what the attention kernel holds per lane (1024)"; return nullptr; }
             L.scale = (float)mx["scale"].as_double(1.0);
             const Json &mask = mx["mask"];
             L.window = mask.is_object() ? (int)mask["size"].as_int(0) : 0;
@@ -379,7 +379,6 @@ bool Context::init_novorax(std::string &err) {
     argmax_scratch_ = (float *)dalloc(T * 129 * 4);
     if (!d_argmax_ || !argmax_scratch_ || hipHostMalloc((void **)&h_argmax_, T * 4, hipHostMallocDefault) != hipSuccess) { err = "arg-max buffers allocation failed"; return false; }
     embeddings_enabled = false;
-    cp.use_graphs = false;                                      // the segment lists change the launch shapes from step to step
     kv_clear();
     nvx_state_reset(-1);
     if (hipDeviceSynchronize() != hipSuccess) { err = "device synchronise failed"; return false; }
@@ -439,8 +438,14 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq) {
     return hipMemcpyAsync(d_seg_, h_seg_, 3 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
 }
 
-hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale) {
+// pn != nullptr: the rows of x are RMS-normed with weight (1 + pn) on the way in (few rows: inside the launch; batches: a norm launch into xn_ first)
+hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale, const float *pn) {
     MMBArgs a;
+    if (pn && T > MMB_VEC_ROWS) {
+        NVX_TRY(launch_rmsnorm_f32(x, ldx, pn, 1.0f, nullptr, xn_, w.K, w.K, T, model->nvx->eps, stream_));
+        x = xn_; ldx = w.K; pn = nullptr;
+    }
+    a.pn_w = pn; a.pn_off = 1.0f; a.pn_eps = model->nvx->eps;
     a.x = x; a.ldx = ldx; a.w = w.w; a.w2 = w2 ? w2->w : nullptr; a.ldw = w.K; a.y = y; a.ldy = ldy;
     a.T = T; a.N = w.N; a.K = w.K; a.epi = epi; a.f32 = cp.exact_f32 ? 1 : 0; a.out_scale = out_scale;
     return launch_mmb(a, stream_);
@@ -450,7 +455,7 @@ hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width;
     if (L.ff_kind == NVX_FF_DENSE) {
-        NVX_TRY(nvx_linear(L.up, xn_, W, T, nvx_ff_, L.ff, MMB_RELU2));
+        NVX_TRY(nvx_linear(L.up, x_, W, T, nvx_ff_, L.ff, MMB_RELU2, nullptr, 1.0f, L.norm2));
         NVX_TRY(nvx_linear(L.down_ff, nvx_ff_, L.ff, T, nvx_y_, W));
         return hipSuccess;
     }
@@ -463,6 +468,8 @@ hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
     d.w = L.e_down.w; d.ldw = L.ff; d.N = W; d.K = L.ff; d.f32 = g.f32; d.w_zs = (long long)W * L.ff;
     d.x = nvx_ff_; d.ldx = L.ff; d.y = nvx_yg_; d.ldy = W;
     const bool grouped = P > 32 && NE <= 64 && (size_t)P * 4 <= 60 * 1024;
+    const bool fuse_norm = !grouped && T <= MMB_VEC_ROWS;         // the pair products norm their row themselves
+    if (!fuse_norm) NVX_TRY(launch_rmsnorm_f32(x_, W, L.norm2, 1.0f, nullptr, xn_, W, W, T, M.eps, stream_));
     if (grouped) {
         // every expert sees its (token, rank) pairs as one batch of rows: counting sort by expert, gather, two grouped products, combine per token
         NVX_TRY(launch_moe_group(nvx_ids_, T, k, NE, nvx_meta_, nvx_slot_, nvx_tokof_, stream_));
@@ -474,7 +481,8 @@ hipError_t Context::nvx_feed_forward(const NvxLayer &L, int T) {
         NVX_TRY(launch_moe_uniform_combine(nvx_y_, nvx_yg_, nvx_slot_, T, W, k, 1.0f / (float)k, stream_));
     } else {
         // a few tokens: one product per (token, rank) pair against the weights the pair picked
-        g.x = xn_; g.ldx = W; g.T = 1; g.nz = P; g.sel = nvx_ids_; g.sel_div = k;
+        g.x = fuse_norm ? x_ : xn_; g.ldx = W; g.T = 1; g.nz = P; g.sel = nvx_ids_; g.sel_div = k;
+        if (fuse_norm) { g.pn_w = L.norm2; g.pn_off = 1.0f; g.pn_eps = M.eps; }
         d.T = 1; d.nz = P; d.sel = nvx_ids_; d.sel_div = 1;
         NVX_TRY(launch_mmb(g, stream_));
         NVX_TRY(launch_mmb(d, stream_));
@@ -501,12 +509,11 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(nvx_linear(M.loop_in, nvx_xcat_, 2 * W, T, x_, W));
             NVX_TRY(launch_add_row(x_, M.loop_step + (size_t)r.pass * W, W, T, stream_));
         }
-        NVX_TRY(launch_rmsnorm_f32(x_, W, L.norm1, 1.0f, nullptr, xn_, W, W, T, eps, stream_));
         const int H = L.heads;
         if (L.type == NVX_LATENT) {
             const int QD = L.dim + L.rot, KR = L.kv_rank, LD_A = L.q_rank + KR + L.rot;
             float *cache = nvx_cache_[(size_t)r.plane];
-            NVX_TRY(nvx_linear(L.down, xn_, W, T, nvx_a_, LD_A));
+            NVX_TRY(nvx_linear(L.down, x_, W, T, nvx_a_, LD_A, MMB_STORE, nullptr, 1.0f, L.norm1));
             LatentPrepArgs pa{};
             pa.a = nvx_a_; pa.ld_a = LD_A; pa.T = T; pa.q_rank = L.q_rank; pa.kv_rank = KR; pa.rot = L.rot; pa.rot_dims = L.rot_dims;
             pa.wq_norm = L.dq_norm; pa.wkv_norm = L.dkv_norm; pa.eps = eps; pa.rot_freq = L.rot_freq; pa.rot_mscale = L.rot_mscale;
@@ -531,7 +538,7 @@ hipError_t Context::run_layers_novorax(int T) {
             prof_mark("latent_attention");
         } else {
             const int LD_P = L.proj.N;
-            NVX_TRY(nvx_linear(L.proj, xn_, W, T, nvx_a_, LD_P));
+            NVX_TRY(nvx_linear(L.proj, x_, W, T, nvx_a_, LD_P, MMB_STORE, nullptr, 1.0f, L.norm1));
             MlstmArgs ma{};
             ma.p = nvx_a_; ma.ld_p = LD_P; ma.o = nvx_o_; ma.ld_o = H * L.vdim; ma.H = H; ma.D = L.dim; ma.VD = L.vdim; ma.gate_cap = L.gate_cap;
             ma.i_bias = L.i_bias; ma.f_bias = L.f_bias; ma.S = nvx_S_[(size_t)r.plane]; ma.n = nvx_n_[(size_t)r.plane]; ma.m = nvx_m_[(size_t)r.plane];
@@ -546,7 +553,6 @@ hipError_t Context::run_layers_novorax(int T) {
         }
         NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));
         if (L.ff_kind != NVX_FF_NONE) {
-            NVX_TRY(launch_rmsnorm_f32(x_, W, L.norm2, 1.0f, nullptr, xn_, W, W, T, eps, stream_));
             NVX_TRY(nvx_feed_forward(L, T));
             NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm2b, 1.0f, x_, x_, W, W, T, eps, stream_));
             prof_mark("feed_forward");
@@ -564,9 +570,8 @@ hipError_t Context::run_output_novorax(int n_out, int out_base) {
     const int W = M.width, V = M.n_vocab;
     float *const xo = cur_T_ == 1 && n_out == 1 ? x_ : xo_;
     if (xo != x_) NVX_TRY(launch_gather_rows_f32(x_, d_outrow_, n_out, W, xo_, stream_));
-    NVX_TRY(launch_rmsnorm_f32(xo, W, M.final_norm, 1.0f, nullptr, xn_, W, W, n_out, M.eps, stream_));
     float *lg = d_logits_ + (size_t)out_base * V;
-    NVX_TRY(nvx_linear(M.head, xn_, W, n_out, lg, V, MMB_STORE, nullptr, M.logit_scale));
+    NVX_TRY(nvx_linear(M.head, xo, W, n_out, lg, V, MMB_STORE, nullptr, M.logit_scale, M.final_norm));
     prof_mark("lm_head");
     for (int r0 = 0; r0 < n_out; r0 += (int)cp.n_ubatch) {
         const int nr = std::min((int)cp.n_ubatch, n_out - r0);

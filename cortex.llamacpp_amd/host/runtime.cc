@@ -1941,28 +1941,21 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
     if (stage_event_) (void)hipEventRecord(stage_event_, stream_);
 
     const int V = model->hp.n_vocab;
-    if (model->nvx) {
-        if (ub_embd_) { last_error = "a Novorax model takes token ids, not embeddings"; return -1; }
-        prof_begin();
-        hipError_t en = run_layers_novorax(n);
-        if (en == hipSuccess) en = run_output_novorax(n_out, out_base);
-        if (en == hipSuccess && n_out > 0 && cp.logits_to_host)
-            en = hipMemcpyAsync(h_logits_ + (size_t)out_base * V, d_logits_ + (size_t)out_base * V, (size_t)n_out * V * 4, hipMemcpyDeviceToHost, stream_);
-        prof_end();
-        if (en != hipSuccess) { last_error = std::string("decode failed: ") + hipGetErrorString(en) + " / " + last_error_string(); return -1; }
-        dbg_tokens_ = n;
-        return 0;
-    }
-    if (n == 1 && !model->hp.encoder && !ub_embd_) { (void)mega_prepare(); (void)engine_prepare(); }   // allocate and upload on first use: must not happen inside a stream capture
+    const bool nvx = model->nvx != nullptr;
+    if (nvx && ub_embd_) { last_error = "a Novorax model takes token ids, not embeddings"; return -1; }
+    const auto layers_of = [&](int T, int cap) { return nvx ? run_layers_novorax(T) : run_layers(T, cap); };
+    const auto output_of = [&](int rows, int base) { return nvx ? run_output_novorax(rows, base) : run_output(rows, base); };
+    if (n == 1 && !model->hp.encoder && !ub_embd_ && !nvx) { (void)mega_prepare(); (void)engine_prepare(); }   // allocate and upload on first use: must not happen inside a stream capture
     // a single-token step would launch the attention + attn_output kernel whose workgroups wait for each other: only while no other context of this device has
     // such a step in flight (runtime.h fused_acquire); otherwise this step takes the wait-free launches, eagerly (the captured graphs hold the fused kernel)
-    attn_out_skip_step_ = n == 1 && !attn_out_off_ && !model->hp.encoder && !fused_acquire();
+    attn_out_skip_step_ = n == 1 && !attn_out_off_ && !model->hp.encoder && !nvx && !fused_acquire();
     if (attn_out_skip_step_) fused_skipped_steps++;
     bool graph_ok = cp.use_graphs && n == 1 && n_out == 1 && out_base == 0 && !profile_ && !debug_taps_ && !embeddings_enabled && moe_forced_T_ == 0 && !ub_embd_ && !attn_out_skip_step_;
     hipError_t e = hipSuccess;
     if (graph_ok) {
         // the attention grid is sized for an upper bound of occupied cells; one captured graph per 256-cell bucket
         int bucket = std::min((int)cp.n_ctx, (n_kv_ + 255) & ~255);
+        if (nvx) bucket = 1 << 30;                             // (no launch of a Novorax step is sized by the cell count: one graph serves every step)
         chunk_cap_ = 0;
         if (chunk_lmax_ > 0) {                                 // chunk lists: the grid is sized by the list length, in steps of 4
             chunk_cap_ = std::min(chunk_stride_, (chunk_lmax_ + 3) & ~3);
@@ -1976,8 +1969,8 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
             e = hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal);
             if (e == hipSuccess) {
                 last_error.clear();
-                hipError_t e2 = run_layers(1, bucket > 0 ? bucket : std::min((int)cp.n_ctx, chunk_cap_ * 64));
-                if (e2 == hipSuccess) e2 = run_output(1, 0);
+                hipError_t e2 = layers_of(1, bucket > 0 ? bucket : std::min((int)cp.n_ctx, chunk_cap_ * 64));
+                if (e2 == hipSuccess) e2 = output_of(1, 0);
                 if (e2 == hipSuccess && cp.logits_to_host && !logits_on_host_) e2 = hipMemcpyAsync(h_logits_, d_logits_, (size_t)V * 4, hipMemcpyDeviceToHost, stream_);
                 if (e2 != hipSuccess) inner = last_error;
                 e = hipStreamEndCapture(stream_, &g);
@@ -2005,8 +1998,8 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
     if (!graph_ok) {
         prof_begin();
         chunk_cap_ = chunk_lmax_;
-        e = run_layers(n, n_kv_);
-        if (e == hipSuccess) e = run_output(n_out, out_base);
+        e = layers_of(n, n_kv_);
+        if (e == hipSuccess) e = output_of(n_out, out_base);
         if (profiler_safe) (void)hipStreamSynchronize(stream_);
         if (e == hipSuccess && n_out > 0 && cp.logits_to_host && !embeddings_enabled && !logits_on_host_)
             e = hipMemcpyAsync(h_logits_ + (size_t)out_base * V, d_logits_ + (size_t)out_base * V, (size_t)n_out * V * 4, hipMemcpyDeviceToHost, stream_);

@@ -180,7 +180,8 @@ class Context {
     bool init_novorax(std::string &err);
     hipError_t run_layers_novorax(int T);
     hipError_t run_output_novorax(int n_out, int out_base);
-    hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f);
+    hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f,
+                          const float *pn = nullptr);
     hipError_t nvx_feed_forward(const NvxLayer &L, int T);
     bool nvx_stage_segments(int n, const int32_t *seq);     // runs of consecutive tokens of one sequence -> segment arrays (pinned, then device)
     void nvx_state_reset(int seq);                          // seq < 0: every slot

@@ -737,6 +737,8 @@ bool LlamaServerContext::UpdateSlots() {   // :1248-1710
                     slot.next_image = 0;
                 }
                 if (prompt_tokens.empty()) prompt_tokens = Tokenize(slot.prompt, be_->vocab().add_bos(), true);
+                // a text without a single token (a tokenizer with no BOS given nothing it knows): one token, so that the request can run at all
+                if (prompt_tokens.empty() && slot.images.empty()) prompt_tokens.push_back(be_->vocab().bos() >= 0 ? be_->vocab().bos() : 0);
                 slot.n_past = 0;
                 slot.num_prompt_tokens = (int32_t)prompt_tokens.size();
                 if (slot.params.n_keep < 0) slot.params.n_keep = slot.num_prompt_tokens;

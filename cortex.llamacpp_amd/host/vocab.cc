@@ -367,8 +367,32 @@ void Vocab::tokenize_wpm(const std::string &text, std::vector<int32_t> &out) con
     }
 }
 
+void Vocab::init_numeric(int n_tokens) {
+    model_ = "numeric";
+    tokens_.resize((size_t)std::max(n_tokens, 0));
+    for (size_t i = 0; i < tokens_.size(); i++) tokens_[i] = std::to_string(i) + " ";
+    scores_.assign(tokens_.size(), 0.0f);
+    types_.assign(tokens_.size(), TT_NORMAL);
+    bos_ = eos_ = eot_ = -1; unk_ = 0;
+    add_bos_ = add_eos_ = add_space_prefix_ = false;
+    index_.clear(); special_ids_.clear(); merge_rank_.clear();
+}
+
 std::vector<int32_t> Vocab::tokenize(const std::string &text, bool add_special, bool parse_special) const {
     std::vector<int32_t> out;
+    if (model_ == "numeric") {
+        for (size_t i = 0; i < text.size();) {
+            if (text[i] < '0' || text[i] > '9') { i++; continue; }
+            const bool word_start = i == 0 || text[i - 1] == ' ' || text[i - 1] == '\n' || text[i - 1] == '\t' || text[i - 1] == ',';
+            size_t j = i;
+            long long v = 0;
+            while (j < text.size() && text[j] >= '0' && text[j] <= '9') { if (v < (1ll << 40)) v = v * 10 + (text[j] - '0'); j++; }
+            const bool word_end = j == text.size() || text[j] == ' ' || text[j] == '\n' || text[j] == '\t' || text[j] == ',';
+            if (word_start && word_end && v < (long long)tokens_.size()) out.push_back((int32_t)v);
+            i = j;
+        }
+        return out;
+    }
     if (model_ == "bert") {
         if (add_special) out.push_back(cls_);
         tokenize_wpm(text, out);
@@ -421,6 +445,7 @@ std::vector<int32_t> Vocab::tokenize(const std::string &text, bool add_special, 
 std::string Vocab::token_to_piece(int32_t id, bool special) const {
     if (id < 0 || id >= n_tokens()) return "";
     const std::string &t = tokens_[(size_t)id];
+    if (model_ == "numeric") return t;
     const int ty = types_[(size_t)id];
     if (ty == TT_CONTROL || ty == TT_UNKNOWN) return special ? t : "";
     if (model_ == "gpt2") {

@@ -30,6 +30,9 @@ class Vocab {
                   int bos, int eos, int unk, bool add_bos);
 
     void init_wpm(const std::vector<std::string> &tokens, int cls, int sep, int unk);      // a "bert" vocabulary (tests)
+    // a model that ships no tokenizer (a folder of config.json + safetensors): text is a list of decimal token ids separated by blanks, token i prints as
+    // "i " - requests and answers stay readable, and the engine's text surface works unchanged.  No bos / eos; words that are not ids in range are skipped.
+    void init_numeric(int n_tokens);
 
     int n_tokens() const { return (int)tokens_.size(); }
     int bos() const { return bos_; }
