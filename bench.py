@@ -227,8 +227,87 @@ def simulate(args) -> int:
     return 0
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / f16 matrix-core peak of MI355X
+
+
+def _time_model(pkg, model, ctx_kw, prompt_len, steps, warmup, n_vocab, seed=1):
+    """Prefill of one prompt and single-token steps behind it on a fresh context: (prefill tok/s, decode tok/s, ms per step)."""
+    rng = np.random.default_rng(seed)
+    toks = rng.integers(0, n_vocab, prompt_len + steps + warmup + 1).astype(np.int32)
+    ctx = pkg.Context(model, **ctx_kw)
+    ctx.decode(toks[:prompt_len], np.arange(prompt_len))          # untimed: first-use allocations, code upload
+    ctx.logits_ready()
+    ctx.kv_clear()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    ctx.decode(toks[:prompt_len], np.arange(prompt_len))
+    ctx.logits_ready()
+    dt_p = time.perf_counter() - t0
+    pos = prompt_len
+    for _ in range(warmup):
+        ctx.decode(toks[pos:pos + 1], [pos]); ctx.logits_ready(); pos += 1
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.decode(toks[pos:pos + 1], [pos]); ctx.logits_ready(); pos += 1
+    dt_d = time.perf_counter() - t0
+    ctx.close()
+    return prompt_len / dt_p, steps / dt_d, dt_d / steps * 1e3
+
+
+def novorax_section(args) -> int:
+    """--novorax SIZES: prefill and decode throughput of synthetic Novorax models (bf16 weights, serving precision) beside the closest model this backend
+    already had - a Llama graph with F16 weights of the same width, depth, dense feed-forward width and vocabulary - with each side's distance from its
+    roofline: prefill as a fraction of the dense 16-bit matrix-core peak (2 FLOP per active weight and token), decode as a fraction of the HBM peak (weight
+    bytes one token reads).  One JSON line; the default workload of this script is untouched."""
+    import __graft_entry__ as ge
+    pkg = ge.load_pkg()
+    pkg.Backend()
+    ns, gs = pkg.novorax_synth, pkg.gguf_synth
+    rows = []
+    for size in [x for x in args.novorax.split(",") if x]:
+        s = ns.SIZES[size]
+        folder = os.path.join(args.model_dir, f"mi355-bench-novorax-{size}")
+        if not os.path.exists(os.path.join(folder, "model.safetensors")):
+            ns.write_synthetic_novorax(folder, size, seed=0xC0FFEE)
+        cfg = ns.config_of(s)
+        wbytes = ns.weight_bytes_per_token(cfg)
+        flops_tok = wbytes - 2 * s.width                     # 2 FLOP per active weight = its bf16 bytes (the embedding row is a lookup)
+        kw = dict(n_ctx=args.ctx, n_batch=N_UBATCH, n_ubatch=N_UBATCH, n_seq_max=1)
+        m = pkg.Model(folder)
+        pf, dc, ms = _time_model(pkg, m, kw, args.prompt, args.steps, args.warmup, s.vocab)
+        m.close()
+        row = {"size": size, "width": s.width, "layers": len(cfg["layers"]), "prompt": args.prompt,
+               "novorax": {"prefill_tok_s": round(pf, 1), "decode_tok_s": round(dc, 2), "ms_per_step": round(ms, 4), "weight_bytes_per_token": wbytes,
+                           "prefill_frac_of_mfma_peak": round(pf * flops_tok / (MFMA_BF16_PEAK_TFLOPS * 1e12), 4),
+                           "decode_frac_of_hbm_peak": round(wbytes * dc / (HBM_PEAK_GBPS * 1e9), 4)}}
+        lc = gs.LlamaConfig(f"f16-twin-{size}", s.width, len(cfg["layers"]), s.width // 128, s.width // 128, s.ff, s.vocab, 500000.0, 1e-5, args.ctx)
+        path = os.path.join(args.model_dir, f"mi355-bench-f16-twin-{size}.gguf")
+        if not os.path.exists(path):
+            gs.write_synthetic_llama(path + ".tmp", lc, "f16", seed=0xC0FFEE, with_vocab=False)
+            os.replace(path + ".tmp", path)
+        m = pkg.Model(path)
+        lb = int(m.bytes_per_token)
+        pf2, dc2, ms2 = _time_model(pkg, m, dict(kw, type_k=pkg.binding.F16, type_v=pkg.binding.F16), args.prompt, args.steps, args.warmup, s.vocab)
+        m.close()
+        row["llama_f16"] = {"prefill_tok_s": round(pf2, 1), "decode_tok_s": round(dc2, 2), "ms_per_step": round(ms2, 4), "weight_bytes_per_token": lb,
+                            "prefill_frac_of_mfma_peak": round(pf2 * lb / (MFMA_BF16_PEAK_TFLOPS * 1e12), 4),
+                            "decode_frac_of_hbm_peak": round(lb * dc2 / (HBM_PEAK_GBPS * 1e9), 4)}
+        a, b = row["novorax"], row["llama_f16"]
+        row["roofline_ratio"] = {"prefill": round(a["prefill_frac_of_mfma_peak"] / max(b["prefill_frac_of_mfma_peak"], 1e-9), 3),
+                                 "decode": round(a["decode_frac_of_hbm_peak"] / max(b["decode_frac_of_hbm_peak"], 1e-9), 3)}
+        rows.append(row)
+        if not args.keep_model:
+            for f in (path, os.path.join(folder, "model.safetensors"), os.path.join(folder, "config.json")):
+                if os.path.exists(f):
+                    os.remove(f)
+    print(json.dumps({"metric": "novorax_prefill_decode_tok_s_vs_f16_llama", "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "dtype": "bf16", "data": "synthetic", "higher_is_better": True, "sizes": rows}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--novorax", default="", help="comma list of synthetic Novorax sizes (w1024, w2048, w4096): time them beside an F16 Llama twin and exit")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -268,6 +347,8 @@ def main() -> int:
         return 2
     if args.simulate:
         return simulate(args)
+    if args.novorax:
+        return novorax_section(args)
 
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

@@ -21,6 +21,7 @@
 #include "../../cortex.llamacpp_amd/host/grammar.h"
 #include "../../cortex.llamacpp_amd/host/server_context.h"
 #include "../../cortex.llamacpp_amd/host/vocab.h"
+#include "../../cortex.llamacpp_amd/host/safetensors.h"
 
 using namespace mi355;
 
@@ -1394,6 +1395,61 @@ static int api_shapes_cli() {
 
 static const char *volatile g_stage = "start";
 
+// a model folder without a tokenizer: text is a list of decimal token ids
+static void test_vocab_numeric() {
+    Vocab v;
+    v.init_numeric(500);
+    CHECK(v.n_tokens() == 500 && v.bos() < 0 && v.eos() < 0 && !v.add_bos() && v.has_vocab());
+    CHECK((v.tokenize("5 17 3", true) == std::vector<int32_t>{5, 17, 3}));
+    CHECK((v.tokenize("u: 5,17\n499 500 12a a7 0", true, true) == std::vector<int32_t>{5, 17, 499, 0}));   // out of range and mixed words are skipped
+    CHECK(v.tokenize("hello", true).empty());
+    CHECK(v.token_to_piece(42) == "42 " && v.detokenize({1, 22, 333}) == "1 22 333 ");
+    CHECK(v.tokenize(v.detokenize({7, 0, 499}), false) == (std::vector<int32_t>{7, 0, 499}));
+    for (int id = 0; id < 500; id++) CHECK(!v.is_eog(id));
+}
+
+// the safetensors reader: header arithmetic, every range checked against the file
+static void test_safetensors_reader() {
+    char tmpl[] = "/tmp/mi355_st_XXXXXX";
+    const int fd = mkstemp(tmpl);
+    CHECK(fd >= 0);
+    auto write_file = [&](const std::string &head, size_t data_bytes, uint64_t claimed = 0) {
+        FILE *f = fopen(tmpl, "wb");
+        uint64_t n = claimed ? claimed : head.size();
+        for (int i = 0; i < 8; i++) fputc((int)((n >> (8 * i)) & 0xff), f);
+        fwrite(head.data(), 1, head.size(), f);
+        for (size_t i = 0; i < data_bytes; i++) fputc((int)(i & 0xff), f);
+        fclose(f);
+    };
+    {
+        write_file("{\"a\":{\"dtype\":\"BF16\",\"shape\":[2,3],\"data_offsets\":[0,12]},\"t\":{\"dtype\":\"I32\",\"shape\":[2],\"data_offsets\":[12,20]},\"__metadata__\":{\"k\":\"v\"}}", 20);
+        SafeTensorsFile st;
+        CHECK(st.open(tmpl).empty());
+        const SafeTensor *a = st.find("a"), *t = st.find("t");
+        CHECK(a && t && !st.find("__metadata__") && !st.find("b"));
+        CHECK(a && a->dtype == "BF16" && a->shape == (std::vector<int64_t>{2, 3}) && a->bytes == 12 && a->data[1] == 1);
+        CHECK(t && t->data[0] == 12 && t->numel() == 2);
+    }
+    const char *bad[] = {
+        "{\"a\":{\"dtype\":\"BF16\",\"shape\":[2,3],\"data_offsets\":[0,40]}}",        // beyond the file
+        "{\"a\":{\"dtype\":\"BF16\",\"shape\":[2,4],\"data_offsets\":[0,12]}}",        // shape against byte range
+        "{\"a\":{\"dtype\":\"Q9\",\"shape\":[12],\"data_offsets\":[0,12]}}",           // unknown dtype
+        "{\"a\":{\"dtype\":\"BF16\",\"shape\":[-6],\"data_offsets\":[0,12]}}",         // negative dimension
+        "{\"a\":{\"dtype\":\"BF16\",\"shape\":[6],\"data_offsets\":[8,2]}}",           // reversed range
+        "[1,2,3]",
+    };
+    for (const char *h : bad) {
+        write_file(h, 20);
+        SafeTensorsFile st;
+        CHECK(!st.open(tmpl).empty());
+    }
+    { write_file("{}", 4, 1ull << 40); SafeTensorsFile st; CHECK(!st.open(tmpl).empty()); }     // header length beyond the file
+    { FILE *f = fopen(tmpl, "wb"); fputc(1, f); fclose(f); SafeTensorsFile st; CHECK(!st.open(tmpl).empty()); }
+    { SafeTensorsFile st; CHECK(st.open("/nonexistent/x.safetensors").rfind("cannot", 0) == 0); }
+    close(fd);
+    unlink(tmpl);
+}
+
 int main(int argc, char **argv) {
     if (argc == 4 && std::string(argv[1]) == "--tokenize") return tokenize_cli(argv[2], argv[3]);
     if (argc == 2 && std::string(argv[1]) == "--api-shapes") return api_shapes_cli();
@@ -1403,6 +1459,8 @@ int main(int argc, char **argv) {
     STAGE(test_json);
     STAGE(test_vocab);
     STAGE(test_vocab_wordpiece);
+    STAGE(test_vocab_numeric);
+    STAGE(test_safetensors_reader);
     STAGE(test_sampler);
     STAGE(test_sampler_topk_matches_full_sort);
     STAGE(test_sampler_mirostat_dynatemp);
