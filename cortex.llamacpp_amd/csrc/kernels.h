@@ -322,6 +322,8 @@ struct MlstmArgs {
     const int32_t *seg_start, *seg_len, *seg_slot; int n_seg;   // runs of consecutive batch rows of one sequence each; no slot twice in a launch
 };
 bool mlstm_shape_ok(int D, int VD);
+// the i / f columns of p become the log gates, in place (biases and the cap applied): once per batch, before the scans
+hipError_t launch_mlstm_gates(const MlstmArgs &a, int T, hipStream_t st);
 hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st);
 // y[t][h][j] = o / rms(o over the head) * w[h][j] * sigmoid(p[t][off_g + h * VD + j])
 hipError_t launch_mlstm_out(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int T, int H, int VD, float eps, float *y, int ld_y,

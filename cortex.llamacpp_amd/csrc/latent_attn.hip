@@ -64,78 +64,141 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(LatentPrepArgs a) {
     }
 }
 
-constexpr int LA_MAX_ACC = 16;                                  // latent values per lane: kv_rank <= 1024
+constexpr int LA_MAX_L = 1088;                                  // kv_rank + rot the attention kernel is instantiated for (17 x 64)
 
-// one workgroup per (token, head); its four waves take every fourth cell of the scanned range and keep their own running maximum, sum and weighted latent,
-// merged at the end together with the sink term
-__global__ __launch_bounds__(256) void latent_attn_kernel(LatentAttnArgs a) {
+// One workgroup per (token, head), NW waves.  A wave works on four cells at a time: each 16-lane group owns one cell, its lanes hold the row's elements
+// 64 j + 4 li .. + 3 (16-byte loads, the whole group reads 256 contiguous bytes per j) and the matching running sums; the next four cells of the wave are
+// requested before the current ones are used.  Every group keeps its own running maximum / sum / weighted latent; groups, then waves, are merged at the
+// end together with the sink term.  NJ = ceil((kv_rank + rot) / 64); VEC: rows are 16-byte aligned (kv_rank + rot a multiple of 4).
+template <int NJ, bool VEC>
+__global__ __launch_bounds__(512) void latent_attn_kernel(LatentAttnArgs a) {
     extern __shared__ float lds[];
-    const int KR = a.kv_rank, R = a.rot, L = KR + R;
-    float *qv = lds;                                            // [L]
-    float *wm = lds + L, *wl = wm + 4, *wacc = wl + 4;           // [4], [4], [4][KR]
-    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int KR = a.kv_rank, R = a.rot, L = KR + R, LP = NJ * 64;
+    const int NW = blockDim.x >> 6;
+    float *qv = lds;                                            // [LP] (zero beyond L)
+    float *wm = lds + LP, *wl = wm + NW, *wacc = wl + NW;        // [NW], [NW], [NW][LP]
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, li = lane & 15;
     const int tpos = a.tok_pos[t];
     const uint64_t sbit = 1ull << (a.tok_seq[t] & 63);
-    for (int i = tid; i < KR; i += 256) qv[i] = a.qa[(size_t)t * a.ld_qa + (size_t)h * KR + i];
-    {
-        const float *qr = a.q + (size_t)t * a.ld_q + (size_t)h * (a.dim + R) + a.dim;
-        const float p = (float)tpos;
-        for (int i = tid; i < R; i += 256) {
-            if (i < a.rot_dims) {
-                const int pr = i >> 1;
-                const float ang = p * a.rot_freq[pr], c = cosf(ang) * a.rot_mscale, s = sinf(ang) * a.rot_mscale;
-                const float u = qr[2 * pr], v = qr[2 * pr + 1];
-                qv[KR + i] = (i & 1) ? v * c + u * s : u * c - v * s;
-            } else qv[KR + i] = qr[i];
+    for (int i = tid; i < LP; i += blockDim.x) {
+        float v = 0.0f;
+        if (i < KR) v = a.qa[(size_t)t * a.ld_qa + (size_t)h * KR + i];
+        else if (i < L) {
+            const float *qr = a.q + (size_t)t * a.ld_q + (size_t)h * (a.dim + R) + a.dim;
+            const int r = i - KR;
+            if (r < a.rot_dims) {
+                const int pr = r >> 1;
+                const float ang = (float)tpos * a.rot_freq[pr], c = cosf(ang) * a.rot_mscale, sn = sinf(ang) * a.rot_mscale;
+                const float u = qr[2 * pr], w = qr[2 * pr + 1];
+                v = (r & 1) ? w * c + u * sn : u * c - w * sn;
+            } else v = qr[r];
         }
+        qv[i] = v;
     }
     __syncthreads();
-    const int nacc = (KR + 63) >> 6, nall = (L + 63) >> 6;
-    float acc[LA_MAX_ACC];
+    float acc[NJ][4], cur[NJ][4], nxt[NJ][4];
 #pragma unroll
-    for (int j = 0; j < LA_MAX_ACC; j++) acc[j] = 0.0f;
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) { acc[j][e] = 0.0f; cur[j][e] = 0.0f; nxt[j][e] = 0.0f; }
     float m = -INFINITY, l = 0.0f;
-    const int n_kv = *a.n_kv_dev;
-    for (int c = wave; c < n_kv; c += 4) {
+    const int n_kv = *a.n_kv_dev, stride = NW * 4;
+    const auto visible = [&](int c) {
+        if (c >= n_kv) return false;
         const int cp = a.cell_pos[c];
-        if (cp < 0 || cp > tpos || !(a.cell_seq[c] & sbit) || (a.window > 0 && tpos - cp >= a.window)) continue;   // (wave-uniform)
+        return cp >= 0 && cp <= tpos && (a.cell_seq[c] & sbit) != 0 && !(a.window > 0 && tpos - cp >= a.window);
+    };
+    const auto fetch = [&](int c, bool vis, float (&dst)[NJ][4]) {
         const float *row = a.cache + (size_t)c * L;
-        float vals[LA_MAX_ACC], dot = 0.0f;
 #pragma unroll
-        for (int j = 0; j < LA_MAX_ACC; j++) {
-            vals[j] = 0.0f;
-            if (j < nacc && j * 64 + lane < KR) { vals[j] = row[j * 64 + lane]; dot = fmaf(vals[j], qv[j * 64 + lane], dot); }
+        for (int j = 0; j < NJ; j++) {
+            const int e0 = 64 * j + 4 * li;
+            if (VEC) {
+                float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (vis && e0 < L) v = *reinterpret_cast<const float4 *>(row + e0);
+                dst[j][0] = v.x; dst[j][1] = v.y; dst[j][2] = v.z; dst[j][3] = v.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) dst[j][e] = vis && e0 + e < L ? row[e0 + e] : 0.0f;
+            }
         }
-        for (int i = KR + lane; i < L; i += 64) dot = fmaf(row[i], qv[i], dot);
-        (void)nall;
-        const float s = wave_sum(dot) * a.scale;
-        const float mn = fmaxf(m, s), alpha = expf(m - mn), p = expf(s - mn);   // (m = -inf at the first visible cell: alpha = 0)
-        l = l * alpha + p;
+    };
+    int c = wave * 4 + g;
+    bool vis = visible(c);
+    fetch(c, vis, cur);
+    for (int c0 = 0; c0 < n_kv; c0 += stride) {                 // (uniform trip count: the shuffles below are executed by whole waves)
+        const int cn = c + stride;
+        const bool visn = visible(cn);
+        fetch(cn, visn, nxt);
+        float dot = 0.0f;
 #pragma unroll
-        for (int j = 0; j < LA_MAX_ACC; j++) acc[j] = acc[j] * alpha + p * vals[j];
-        m = mn;
+        for (int j = 0; j < NJ; j++) {
+            const float4 q4 = *reinterpret_cast<const float4 *>(qv + 64 * j + 4 * li);
+            dot = fmaf(cur[j][0], q4.x, dot); dot = fmaf(cur[j][1], q4.y, dot); dot = fmaf(cur[j][2], q4.z, dot); dot = fmaf(cur[j][3], q4.w, dot);
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+        if (vis) {
+            const float sc = dot * a.scale;
+            const float mn = fmaxf(m, sc), alpha = expf(m - mn), p = expf(sc - mn);   // (m = -inf at the group's first cell: alpha = 0)
+            l = l * alpha + p;
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[j][e] = acc[j][e] * alpha + p * cur[j][e];
+            m = mn;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) cur[j][e] = nxt[j][e];
+        c = cn; vis = visn;
     }
-    if (lane == 0) { wm[wave] = m; wl[wave] = l; }
+    // the four groups of a wave -> one record per wave
+    float M = fmaxf(m, __shfl_xor(m, 16, 64));
+    M = fmaxf(M, __shfl_xor(M, 32, 64));
+    const float sg = l > 0.0f ? expf(m - M) : 0.0f;
+    l *= sg;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
 #pragma unroll
-    for (int j = 0; j < LA_MAX_ACC; j++)
-        if (j < nacc && j * 64 + lane < KR) wacc[wave * KR + j * 64 + lane] = acc[j];
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float v = acc[j][e] * sg;
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            if (g == 0) wacc[wave * LP + 64 * j + 4 * li + e] = v;
+        }
+    if (lane == 0) { wm[wave] = M; wl[wave] = l; }
     __syncthreads();
-    float M = fmaxf(fmaxf(wm[0], wm[1]), fmaxf(wm[2], wm[3]));
-    const float sink = a.sink ? a.sink[h] : -INFINITY;
-    M = fmaxf(M, sink);
-    float sc[4], den = a.sink ? expf(sink - M) : 0.0f;
-#pragma unroll
-    for (int w = 0; w < 4; w++) { sc[w] = wl[w] > 0.0f ? expf(wm[w] - M) : 0.0f; den += wl[w] * sc[w]; }
+    float MM = a.sink ? a.sink[h] : -INFINITY;
+    for (int w = 0; w < NW; w++) MM = fmaxf(MM, wm[w]);
+    float den = a.sink ? expf(a.sink[h] - MM) : 0.0f;
+    for (int w = 0; w < NW; w++) den += wl[w] > 0.0f ? wl[w] * expf(wm[w] - MM) : 0.0f;
     const float inv = den > 0.0f ? 1.0f / den : 0.0f;
-    for (int i = tid; i < KR; i += 256) {
-        const float o = wacc[i] * sc[0] + wacc[KR + i] * sc[1] + wacc[2 * KR + i] * sc[2] + wacc[3 * KR + i] * sc[3];
+    for (int i = tid; i < KR; i += blockDim.x) {
+        float o = 0.0f;
+        for (int w = 0; w < NW; w++) o += wl[w] > 0.0f ? wacc[w * LP + i] * expf(wm[w] - MM) : 0.0f;
         a.out[(size_t)t * a.ld_out + (size_t)h * KR + i] = o * inv;
     }
 }
 
+template <int NJ>
+static hipError_t launch_latent_attn_nj(const LatentAttnArgs &a, hipStream_t st) {
+    // few (token, head) pairs - single-token steps - get eight waves each: more cells in flight where the grid alone cannot fill the device
+    const int nw = (long long)a.T * a.H <= 1024 ? 8 : 4;
+    const size_t lds = (size_t)(NJ * 64 + 2 * nw + nw * NJ * 64) * sizeof(float);
+    const bool vec = ((a.kv_rank + a.rot) & 3) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0;
+    const dim3 grid((unsigned)a.T, (unsigned)a.H);
+    if (vec) hipLaunchKernelGGL((latent_attn_kernel<NJ, true>), grid, dim3(64 * nw), lds, st, a);
+    else hipLaunchKernelGGL((latent_attn_kernel<NJ, false>), grid, dim3(64 * nw), lds, st, a);
+    return hipGetLastError();
+}
+
 }  // namespace
 
-bool latent_attn_shape_ok(int kv_rank, int rot) { return kv_rank >= 1 && kv_rank <= 64 * LA_MAX_ACC && rot >= 0 && rot <= 4096; }
+bool latent_attn_shape_ok(int kv_rank, int rot) { return kv_rank >= 1 && rot >= 0 && kv_rank + rot <= LA_MAX_L; }
 
 hipError_t launch_latent_prep(const LatentPrepArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
@@ -147,9 +210,11 @@ hipError_t launch_latent_prep(const LatentPrepArgs &a, hipStream_t st) {
 hipError_t launch_latent_attn(const LatentAttnArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
     if (!latent_attn_shape_ok(a.kv_rank, a.rot) || a.rot_dims > a.rot || (a.rot_dims & 1)) return hipErrorInvalidValue;
-    const size_t lds = (size_t)(a.kv_rank + a.rot + 8 + 4 * a.kv_rank) * sizeof(float);
-    hipLaunchKernelGGL(latent_attn_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), lds, st, a);
-    return hipGetLastError();
+    const int L = a.kv_rank + a.rot;
+    if (L <= 128) return launch_latent_attn_nj<2>(a, st);
+    if (L <= 320) return launch_latent_attn_nj<5>(a, st);
+    if (L <= 576) return launch_latent_attn_nj<9>(a, st);
+    return launch_latent_attn_nj<17>(a, st);
 }
 
 }  // namespace mi355

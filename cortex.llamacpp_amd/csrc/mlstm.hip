@@ -2,7 +2,7 @@
 //
 // Per head: a state matrix S [dim][vdim], a normaliser n [dim] and a running maximum m of the log gates, all f32, one set per sequence slot.  For a token
 // with query q (already scaled by dim^-1/2 here), key k, value v and the pre-activations of the two gates:
-//     i = cap tanh(i_pre / cap)            f = logsigmoid(cap tanh(f_pre / cap))
+//     i = cap tanh(i_pre / cap)            f = logsigmoid(cap tanh(f_pre / cap))        (both made for the whole batch at once: launch_mlstm_gates)
 //     m' = max(f + m, i)     S' = e^(f + m - m') S + e^(i - m') k v^T     n' likewise with k alone
 //     o  = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6)
 // A state that has seen nothing is S = 0, n = 0, m = 0.  The columns of S evolve independently given the gates, so a workgroup owns 64 columns of one head of
@@ -18,7 +18,7 @@ namespace {
 
 template <int DPER>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
-    __shared__ float sq[256], sk[256], red[4][64], redn[4];
+    __shared__ float sq[4 * DPER], sk[4 * DPER], red[4][64], redn[4];
     const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, j = tid & 63, dg = tid >> 6;
     const int col = blockIdx.z * 64 + j, d0 = dg * DPER;
     const int H = a.H, D = a.D, VD = a.VD;
@@ -34,18 +34,34 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
         n[e] = d < D ? ng[d] : 0.0f;
     }
     float m = *mg;
-    const float qscale = 1.0f / sqrtf((float)D), cap = a.gate_cap;
-    const float ib = a.i_bias ? a.i_bias[h] : 0.0f, fb = a.f_bias ? a.f_bias[h] : 0.0f;
+    const float qscale = 1.0f / sqrtf((float)D);
     const int off_k = H * D, off_v = 2 * H * D, off_i = 2 * H * D + 2 * H * VD, off_f = off_i + H;
-    for (int t = 0; t < len; t++) {
+    // the next token's inputs are requested while the current one is being used (a request per token in the dependency chain would cost a memory
+    // round trip each); the gate columns already hold the log gates (mlstm_gates_kernel)
+    constexpr int NLD = (4 * DPER + 255) / 256;
+    float rq[NLD], rk[NLD], rv, rig, rfg;
+    const auto request = [&](int t) {
         const float *row = a.p + (size_t)(start + t) * a.ld_p;
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int d = tid + 256 * u;
+            rq[u] = d < D ? row[h * D + d] : 0.0f;
+            rk[u] = d < D ? row[off_k + h * D + d] : 0.0f;
+        }
+        rv = col < VD ? row[off_v + h * VD + col] : 0.0f;
+        rig = row[off_i + h];
+        rfg = row[off_f + h];
+    };
+    if (len > 0) request(0);
+    for (int t = 0; t < len; t++) {
         __syncthreads();                                        // (the previous token's partial sums and q / k rows have been read)
-        sq[tid] = tid < D ? row[h * D + tid] * qscale : 0.0f;
-        sk[tid] = tid < D ? row[off_k + h * D + tid] : 0.0f;
-        const float v = col < VD ? row[off_v + h * VD + col] : 0.0f;
-        const float ig = cap * tanhf((row[off_i + h] + ib) / cap);
-        const float fz = cap * tanhf((row[off_f + h] + fb) / cap);
-        const float fg = fminf(fz, 0.0f) - log1pf(expf(-fabsf(fz)));
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int d = tid + 256 * u;
+            if (d < 4 * DPER) { sq[d] = rq[u] * qscale; sk[d] = rk[u]; }
+        }
+        const float v = rv, ig = rig, fg = rfg;
+        if (t + 1 < len) request(t + 1);
         const float mn = fmaxf(fg + m, ig), ea = expf(fg + m - mn), eb = expf(ig - mn);
         m = mn;
         __syncthreads();
@@ -76,6 +92,18 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
     if (blockIdx.z == 0 && tid == 0) *mg = m;
 }
 
+// the two log gates of every (token, head), in place over their pre-activations: i = cap tanh((x + b_i) / cap), f = logsigmoid(cap tanh((x + b_f) / cap))
+__global__ void mlstm_gates_kernel(float *p, int ld_p, int off_i, int H, int T, const float *ib, const float *fb, float cap) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T * H) return;
+    const int t = i / H, h = i - t * H;
+    float *row = p + (size_t)t * ld_p + off_i;
+    const float ig = cap * tanhf((row[h] + (ib ? ib[h] : 0.0f)) / cap);
+    const float fz = cap * tanhf((row[H + h] + (fb ? fb[h] : 0.0f)) / cap);
+    row[h] = ig;
+    row[H + h] = fminf(fz, 0.0f) - log1pf(expf(-fabsf(fz)));
+}
+
 __global__ __launch_bounds__(64) void mlstm_out_kernel(const float *o, int ld_o, const float *p, int ld_p, int off_g, const float *w, int H, int VD, float eps,
                                                        float *y, int ld_y) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -100,7 +128,14 @@ __global__ void mlstm_state_reset_kernel(float *S, size_t n_s, float *n, size_t 
 
 }  // namespace
 
-bool mlstm_shape_ok(int D, int VD) { return D >= 1 && D <= 256 && VD >= 1; }
+bool mlstm_shape_ok(int D, int VD) { return D >= 1 && D <= 512 && VD >= 1; }
+
+hipError_t launch_mlstm_gates(const MlstmArgs &a, int T, hipStream_t st) {
+    if (T <= 0) return hipSuccess;
+    hipLaunchKernelGGL(mlstm_gates_kernel, dim3((unsigned)((T * a.H + 255) / 256)), dim3(256), 0, st, const_cast<float *>(a.p), a.ld_p,
+                       2 * a.H * a.D + 2 * a.H * a.VD, a.H, T, a.i_bias, a.f_bias, a.gate_cap);
+    return hipGetLastError();
+}
 
 hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st) {
     if (a.n_seg <= 0) return hipSuccess;
@@ -109,7 +144,8 @@ hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st) {
     if (a.D <= 32) hipLaunchKernelGGL(mlstm_scan_kernel<8>, grid, dim3(256), 0, st, a);
     else if (a.D <= 64) hipLaunchKernelGGL(mlstm_scan_kernel<16>, grid, dim3(256), 0, st, a);
     else if (a.D <= 128) hipLaunchKernelGGL(mlstm_scan_kernel<32>, grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(mlstm_scan_kernel<64>, grid, dim3(256), 0, st, a);
+    else if (a.D <= 256) hipLaunchKernelGGL(mlstm_scan_kernel<64>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(mlstm_scan_kernel<128>, grid, dim3(256), 0, st, a);
     return hipGetLastError();
 }
 

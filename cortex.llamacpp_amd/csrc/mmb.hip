@@ -55,6 +55,8 @@ __device__ __forceinline__ ZView z_view(const MMBArgs &a, int z) {
 }
 
 // ---------------------------------------------------------------- few rows: one wave per output column
+// With the norm prologue the row's sum of squares is gathered in the same pass as the products: y = inv_rms(x) * sum_k w_k (x_k (off + g_k)) - one trip
+// through memory per wave, the scale applied to the finished sum.
 template <bool VEC>
 __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -62,41 +64,33 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
     const ZView v = z_view(a, blockIdx.y);
     if (n >= a.N) return;
     const unsigned short *wr = v.w + (size_t)n * a.ldw, *wr2 = v.w2 ? v.w2 + (size_t)n * a.ldw : nullptr;
+    const bool pn = a.pn_w != nullptr;
     constexpr int TB = 8;
     for (int t0 = 0; t0 < v.rows; t0 += TB) {
-        float acc[TB], acc2[TB];
+        float acc[TB], acc2[TB], ss[TB];
 #pragma unroll
-        for (int i = 0; i < TB; i++) { acc[i] = 0.0f; acc2[i] = 0.0f; }
+        for (int i = 0; i < TB; i++) { acc[i] = 0.0f; acc2[i] = 0.0f; ss[i] = 0.0f; }
         const int nt = v.rows - t0 < TB ? v.rows - t0 : TB;
-        float inv[TB];                                          // fused RMS norm of the rows: 1 / sqrt(mean(x^2) + eps), every wave for itself
-#pragma unroll
-        for (int i = 0; i < TB; i++) {
-            inv[i] = 1.0f;
-            if (a.pn_w && i < nt) {
-                float ss = 0.0f;
-                for (int k = lane; k < a.K; k += 64) { const float x = v.x[(size_t)(t0 + i) * a.ldx + k]; ss = fmaf(x, x, ss); }
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-                inv[i] = 1.0f / sqrtf(ss / (float)a.K + a.pn_eps);
-            }
-        }
         if (VEC) {
             for (int k = lane * 8; k < a.K; k += 512) {
                 const u16x8 w8 = *reinterpret_cast<const u16x8 *>(wr + k);
                 u16x8 w28 = w8;
                 if (wr2) w28 = *reinterpret_cast<const u16x8 *>(wr2 + k);
                 float pw[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) pw[e] = a.pn_w ? a.pn_off + a.pn_w[k + e] : 1.0f;
+                if (pn) {
+                    const f32x4 g0 = *reinterpret_cast<const f32x4 *>(a.pn_w + k), g1 = *reinterpret_cast<const f32x4 *>(a.pn_w + k + 4);
+                    pw[0] = a.pn_off + g0.x; pw[1] = a.pn_off + g0.y; pw[2] = a.pn_off + g0.z; pw[3] = a.pn_off + g0.w;
+                    pw[4] = a.pn_off + g1.x; pw[5] = a.pn_off + g1.y; pw[6] = a.pn_off + g1.z; pw[7] = a.pn_off + g1.w;
+                }
 #pragma unroll
                 for (int i = 0; i < TB; i++) {
                     if (i >= nt) break;
                     const float *xr = v.x + (size_t)(t0 + i) * a.ldx + k;
                     const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr), x1 = *reinterpret_cast<const f32x4 *>(xr + 4);
                     float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                    if (a.pn_w) {
+                    if (pn) {
 #pragma unroll
-                        for (int e = 0; e < 8; e++) xs[e] = xs[e] * inv[i] * pw[e];
+                        for (int e = 0; e < 8; e++) { ss[i] = fmaf(xs[e], xs[e], ss[i]); xs[e] = xs[e] * pw[e]; }
                     }
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
@@ -107,12 +101,12 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
             }
         } else {
             for (int k = lane; k < a.K; k += 64) {
-                const float w = bf2f(wr[k]), w2 = wr2 ? bf2f(wr2[k]) : 0.0f;
+                const float w = bf2f(wr[k]), w2 = wr2 ? bf2f(wr2[k]) : 0.0f, pw = pn ? a.pn_off + a.pn_w[k] : 1.0f;
 #pragma unroll
                 for (int i = 0; i < TB; i++) {
                     if (i >= nt) break;
                     float x = v.x[(size_t)(t0 + i) * a.ldx + k];
-                    if (a.pn_w) x = x * inv[i] * (a.pn_off + a.pn_w[k]);
+                    if (pn) { ss[i] = fmaf(x, x, ss[i]); x = x * pw; }
                     acc[i] = fmaf(x, w, acc[i]);
                     acc2[i] = fmaf(x, w2, acc2[i]);
                 }
@@ -121,9 +115,10 @@ __global__ __launch_bounds__(256) void mmb_vec_kernel(MMBArgs a) {
 #pragma unroll
         for (int i = 0; i < TB; i++) {
             if (i >= nt) break;
-            float s = acc[i], s2 = acc2[i];
+            float s = acc[i], s2 = acc2[i], q = ss[i];
 #pragma unroll
-            for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o, 64); s2 += __shfl_xor(s2, o, 64); }
+            for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o, 64); s2 += __shfl_xor(s2, o, 64); q += __shfl_xor(q, o, 64); }
+            if (pn) { const float inv = 1.0f / sqrtf(q / (float)a.K + a.pn_eps); s *= inv; s2 *= inv; }
             if (lane == 0) v.y[(size_t)(t0 + i) * a.ldy + n] = epi_apply(a.epi, s, s2) * a.out_scale;
         }
     }
@@ -256,7 +251,7 @@ hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     const auto al = [](const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0; };
     // 16-byte loads of both operands: every row start and every stride on a 16-byte boundary
     const bool vec = (a.K % 8) == 0 && (a.ldw % 8) == 0 && (a.w_zs % 8) == 0 && (a.ldx % 4) == 0 && (a.x_zs % 4) == 0 && al(a.w, 16) && al(a.x, 16) &&
-                     (!a.w2 || al(a.w2, 16));
+                     (!a.w2 || al(a.w2, 16)) && (!a.pn_w || al(a.pn_w, 16));
     const int rows_max = a.sel ? 1 : a.T;                        // most rows any outer index can hold
     if (a.pn_w && rows_max > MMB_VEC_ROWS) return hipErrorInvalidValue;   // (the norm prologue lives in the few-rows kernel only)
     if (rows_max <= MMB_VEC_ROWS || a.sel) {

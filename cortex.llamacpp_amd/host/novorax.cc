@@ -163,7 +163,7 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
             L.type = NVX_LATENT;
             L.rot = (int)mx["rot_dim"].as_int(0); L.kv_rank = (int)mx["kv_rank"].as_int(); L.q_rank = (int)mx["q_rank"].as_int();
             if (!positive(err, "mixer.kv_rank", L.kv_rank) || !positive(err, "mixer.q_rank", L.q_rank) || L.rot < 0) { if (err.empty()) err = "configuration: mixer.rot_dim is negative"; return nullptr; }
-            if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " is beyond what the attention kernel holds per lane (1024)"; return nullptr; }
+            if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " (+ rot_dim) is beyond what the attention kernel holds per lane (1088)"; return nullptr; }
             L.scale = (float)mx["scale"].as_double(1.0);
             const Json &mask = mx["mask"];
             L.window = mask.is_object() ? (int)mask["size"].as_int(0) : 0;
@@ -225,7 +225,7 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
             L.type = NVX_MLSTM;
             L.gate_cap = (float)mx["gate_cap"].as_double(0.0);
             if (!(L.gate_cap > 0.0f)) { err = "configuration: mixer.gate_cap must be positive"; return nullptr; }
-            if (!mlstm_shape_ok(L.dim, L.vdim)) { err = "mlstm: dim " + std::to_string(L.dim) + " is beyond what the recurrence kernel keeps in registers (256)"; return nullptr; }
+            if (!mlstm_shape_ok(L.dim, L.vdim)) { err = "mlstm: dim " + std::to_string(L.dim) + " is beyond what the recurrence kernel keeps in registers (512)"; return nullptr; }
             L.proj = ld.rows({{pm + "q", H * L.dim}, {pm + "k", H * L.dim}, {pm + "v", H * L.vdim}, {pm + "g", H * L.vdim}, {pm + "i", H}, {pm + "f", H}}, W);
             L.i_bias = ld.vec(pm + "i.b", H);
             L.f_bias = ld.vec(pm + "f.b", H);
@@ -542,6 +542,7 @@ hipError_t Context::run_layers_novorax(int T) {
             MlstmArgs ma{};
             ma.p = nvx_a_; ma.ld_p = LD_P; ma.o = nvx_o_; ma.ld_o = H * L.vdim; ma.H = H; ma.D = L.dim; ma.VD = L.vdim; ma.gate_cap = L.gate_cap;
             ma.i_bias = L.i_bias; ma.f_bias = L.f_bias; ma.S = nvx_S_[(size_t)r.plane]; ma.n = nvx_n_[(size_t)r.plane]; ma.m = nvx_m_[(size_t)r.plane];
+            NVX_TRY(launch_mlstm_gates(ma, T, stream_));
             const size_t TU = cp.n_ubatch;
             for (const auto &wv : nvx_waves_) {
                 ma.seg_start = d_seg_ + wv.first; ma.seg_len = d_seg_ + TU + wv.first; ma.seg_slot = d_seg_ + 2 * TU + wv.first; ma.n_seg = wv.second;
