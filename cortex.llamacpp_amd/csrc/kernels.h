@@ -308,7 +308,13 @@ struct LatentAttnArgs {
     int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
     float scale; const float *sink;        // sink: [H] or nullptr
     const float *rot_freq; float rot_mscale;
+    // single-token steps: the scanned cells cut into `splits` runs, one workgroup each, merged afterwards; part: T * H * splits * (kv_rank + 2) floats (nullptr / splits <= 1: one workgroup per (token, head))
+    float *part; int splits;
+    // nullable: per token, one past the highest cell that can hold a key of its sequence at or before its position (host-made from the cell table): the scan
+    // of a prompt's early tokens stops there instead of at the high-water mark
+    const int32_t *tok_hi;
 };
+constexpr int LATENT_ATTN_SPLITS = 8, LATENT_ATTN_SPLIT_MAX_PAIRS = 128;   // (token, head) pairs up to which a step is split
 bool latent_attn_shape_ok(int kv_rank, int rot);
 hipError_t launch_latent_attn(const LatentAttnArgs &a, hipStream_t st);
 

@@ -102,9 +102,19 @@ __global__ __launch_bounds__(512) void latent_attn_kernel(LatentAttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) { acc[j][e] = 0.0f; cur[j][e] = 0.0f; nxt[j][e] = 0.0f; }
     float m = -INFINITY, l = 0.0f;
-    const int n_kv = *a.n_kv_dev, stride = NW * 4;
+    int n_kv = *a.n_kv_dev;
+    if (a.tok_hi) n_kv = a.tok_hi[t] < n_kv ? a.tok_hi[t] : n_kv;
+    const int stride = NW * 4;
+    // gridDim.z > 1 (single-token steps): the scanned range is cut into that many runs of cells, one workgroup each; the runs' records are merged by
+    // latent_attn_merge_kernel
+    int c_lo = 0, c_hi = n_kv;
+    if (gridDim.z > 1) {
+        const int per = ((n_kv + (int)gridDim.z - 1) / (int)gridDim.z + stride - 1) / stride * stride;
+        c_lo = (int)blockIdx.z * per;
+        c_hi = c_lo + per < n_kv ? c_lo + per : n_kv;
+    }
     const auto visible = [&](int c) {
-        if (c >= n_kv) return false;
+        if (c >= c_hi) return false;
         const int cp = a.cell_pos[c];
         return cp >= 0 && cp <= tpos && (a.cell_seq[c] & sbit) != 0 && !(a.window > 0 && tpos - cp >= a.window);
     };
@@ -123,10 +133,10 @@ __global__ __launch_bounds__(512) void latent_attn_kernel(LatentAttnArgs a) {
             }
         }
     };
-    int c = wave * 4 + g;
+    int c = c_lo + wave * 4 + g;
     bool vis = visible(c);
     fetch(c, vis, cur);
-    for (int c0 = 0; c0 < n_kv; c0 += stride) {                 // (uniform trip count: the shuffles below are executed by whole waves)
+    for (int c0 = c_lo; c0 < c_hi; c0 += stride) {              // (uniform trip count: the shuffles below are executed by whole waves)
         const int cn = c + stride;
         const bool visn = visible(cn);
         fetch(cn, visn, nxt);
@@ -172,6 +182,20 @@ __global__ __launch_bounds__(512) void latent_attn_kernel(LatentAttnArgs a) {
         }
     if (lane == 0) { wm[wave] = M; wl[wave] = l; }
     __syncthreads();
+    if (gridDim.z > 1) {                                        // this run's record: maximum, sum, weighted latent (no sink: the merge adds it once)
+        float *rec = a.part + (((size_t)t * a.H + h) * gridDim.z + blockIdx.z) * (size_t)(KR + 2);
+        float Ms = -INFINITY;
+        for (int w = 0; w < NW; w++) if (wl[w] > 0.0f) Ms = fmaxf(Ms, wm[w]);
+        float ls = 0.0f;
+        for (int w = 0; w < NW; w++) ls += wl[w] > 0.0f ? wl[w] * expf(wm[w] - Ms) : 0.0f;
+        if (tid == 0) { rec[0] = Ms; rec[1] = ls; }
+        for (int i = tid; i < KR; i += blockDim.x) {
+            float o = 0.0f;
+            for (int w = 0; w < NW; w++) o += wl[w] > 0.0f ? wacc[w * LP + i] * expf(wm[w] - Ms) : 0.0f;
+            rec[2 + i] = o;
+        }
+        return;
+    }
     float MM = a.sink ? a.sink[h] : -INFINITY;
     for (int w = 0; w < NW; w++) MM = fmaxf(MM, wm[w]);
     float den = a.sink ? expf(a.sink[h] - MM) : 0.0f;
@@ -184,15 +208,32 @@ __global__ __launch_bounds__(512) void latent_attn_kernel(LatentAttnArgs a) {
     }
 }
 
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a, int splits) {
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, KR = a.kv_rank;
+    const float *rec = a.part + ((size_t)t * a.H + h) * splits * (size_t)(KR + 2);
+    float MM = a.sink ? a.sink[h] : -INFINITY;
+    for (int s = 0; s < splits; s++) if (rec[(size_t)s * (KR + 2) + 1] > 0.0f) MM = fmaxf(MM, rec[(size_t)s * (KR + 2)]);
+    float den = a.sink ? expf(a.sink[h] - MM) : 0.0f;
+    for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (KR + 2); den += r[1] > 0.0f ? r[1] * expf(r[0] - MM) : 0.0f; }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    for (int i = tid; i < KR; i += 256) {
+        float o = 0.0f;
+        for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (KR + 2); o += r[1] > 0.0f ? r[2 + i] * expf(r[0] - MM) : 0.0f; }
+        a.out[(size_t)t * a.ld_out + (size_t)h * KR + i] = o * inv;
+    }
+}
+
 template <int NJ>
 static hipError_t launch_latent_attn_nj(const LatentAttnArgs &a, hipStream_t st) {
     // few (token, head) pairs - single-token steps - get eight waves each: more cells in flight where the grid alone cannot fill the device
     const int nw = (long long)a.T * a.H <= 1024 ? 8 : 4;
     const size_t lds = (size_t)(NJ * 64 + 2 * nw + nw * NJ * 64) * sizeof(float);
     const bool vec = ((a.kv_rank + a.rot) & 3) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0;
-    const dim3 grid((unsigned)a.T, (unsigned)a.H);
+    const int splits = a.part && a.splits > 1 ? a.splits : 1;
+    const dim3 grid((unsigned)a.T, (unsigned)a.H, (unsigned)splits);
     if (vec) hipLaunchKernelGGL((latent_attn_kernel<NJ, true>), grid, dim3(64 * nw), lds, st, a);
     else hipLaunchKernelGGL((latent_attn_kernel<NJ, false>), grid, dim3(64 * nw), lds, st, a);
+    if (splits > 1) hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a, splits);
     return hipGetLastError();
 }
 

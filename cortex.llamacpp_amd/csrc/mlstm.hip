@@ -6,7 +6,7 @@
 //     m' = max(f + m, i)     S' = e^(f + m - m') S + e^(i - m') k v^T     n' likewise with k alone
 //     o  = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6)
 // A state that has seen nothing is S = 0, n = 0, m = 0.  The columns of S evolve independently given the gates, so a workgroup owns 64 columns of one head of
-// one sequence segment: lane = column, the four waves split the dim rows (each thread keeps its rows of its column - and of n - in registers), the per-token
+// one sequence segment: lane = column, the 8 or 16 waves split the dim rows (each thread keeps its rows of its column - and of n - in registers), the per-token
 // partial sums of S^T q and n . q cross the waves through LDS.  A segment is a run of consecutive rows of the batch that belong to one sequence: a prompt,
 // a portion of one, or a single decoded token - the same code, started from the slot's state and ending with the state written back.
 // mlstm_out: per head, the output divided by its root mean square, times the mixer's norm weight, times sigmoid of the output gate's pre-activation.
@@ -16,9 +16,12 @@ namespace mi355 {
 
 namespace {
 
-template <int DPER>
-__global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
-    __shared__ float sq[4 * DPER], sk[4 * DPER], red[4][64], redn[4];
+template <int DPER, int NDG>
+__global__ __launch_bounds__(64 * NDG) void mlstm_scan_kernel(MlstmArgs a) {
+    // CH tokens' inputs are staged in LDS by the whole workgroup at once - one trip to memory per CH tokens instead of one per token in the dependency
+    // chain - and the recurrence then runs out of LDS and registers
+    constexpr int DP = NDG * DPER, CH = 2048 / DP, NT = 64 * NDG;
+    __shared__ float sq[CH][DP], sk[CH][DP], sv[CH][64], sg[CH][2], red[2][NDG][64], redn[2][NDG];
     const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, j = tid & 63, dg = tid >> 6;
     const int col = blockIdx.z * 64 + j, d0 = dg * DPER;
     const int H = a.H, D = a.D, VD = a.VD;
@@ -36,51 +39,44 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
     float m = *mg;
     const float qscale = 1.0f / sqrtf((float)D);
     const int off_k = H * D, off_v = 2 * H * D, off_i = 2 * H * D + 2 * H * VD, off_f = off_i + H;
-    // the next token's inputs are requested while the current one is being used (a request per token in the dependency chain would cost a memory
-    // round trip each); the gate columns already hold the log gates (mlstm_gates_kernel)
-    constexpr int NLD = (4 * DPER + 255) / 256;
-    float rq[NLD], rk[NLD], rv, rig, rfg;
-    const auto request = [&](int t) {
-        const float *row = a.p + (size_t)(start + t) * a.ld_p;
-#pragma unroll
-        for (int u = 0; u < NLD; u++) {
-            const int d = tid + 256 * u;
-            rq[u] = d < D ? row[h * D + d] : 0.0f;
-            rk[u] = d < D ? row[off_k + h * D + d] : 0.0f;
+    for (int t0 = 0; t0 < len; t0 += CH) {
+        const int nc = len - t0 < CH ? len - t0 : CH;
+        __syncthreads();                                        // (the previous chunk has been used up)
+        for (int idx = tid; idx < nc * DP; idx += NT) {
+            const int tt = idx / DP, d = idx - tt * DP;
+            const float *row = a.p + (size_t)(start + t0 + tt) * a.ld_p;
+            sq[tt][d] = d < D ? row[h * D + d] * qscale : 0.0f;
+            sk[tt][d] = d < D ? row[off_k + h * D + d] : 0.0f;
         }
-        rv = col < VD ? row[off_v + h * VD + col] : 0.0f;
-        rig = row[off_i + h];
-        rfg = row[off_f + h];
-    };
-    if (len > 0) request(0);
-    for (int t = 0; t < len; t++) {
-        __syncthreads();                                        // (the previous token's partial sums and q / k rows have been read)
-#pragma unroll
-        for (int u = 0; u < NLD; u++) {
-            const int d = tid + 256 * u;
-            if (d < 4 * DPER) { sq[d] = rq[u] * qscale; sk[d] = rk[u]; }
+        for (int idx = tid; idx < nc * 64; idx += NT) {
+            const int tt = idx >> 6, c = blockIdx.z * 64 + (idx & 63);
+            sv[tt][idx & 63] = c < VD ? a.p[(size_t)(start + t0 + tt) * a.ld_p + off_v + h * VD + c] : 0.0f;
         }
-        const float v = rv, ig = rig, fg = rfg;
-        if (t + 1 < len) request(t + 1);
-        const float mn = fmaxf(fg + m, ig), ea = expf(fg + m - mn), eb = expf(ig - mn);
-        m = mn;
+        if (tid < nc * 2) sg[tid >> 1][tid & 1] = a.p[(size_t)(start + t0 + (tid >> 1)) * a.ld_p + ((tid & 1) ? off_f : off_i) + h];   // log gates (mlstm_gates_kernel)
         __syncthreads();
-        float num = 0.0f, nq = 0.0f;
+        for (int tt = 0; tt < nc; tt++) {
+            const float v = sv[tt][j], ig = sg[tt][0], fg = sg[tt][1];
+            const float mn = fmaxf(fg + m, ig), ea = expf(fg + m - mn), eb = expf(ig - mn);
+            m = mn;
+            float num = 0.0f, nq = 0.0f;
 #pragma unroll
-        for (int e = 0; e < DPER; e++) {
-            const float kd = eb * sk[d0 + e], q = sq[d0 + e];
-            S[e] = fmaf(ea, S[e], kd * v);
-            n[e] = fmaf(ea, n[e], kd);
-            num = fmaf(S[e], q, num);
-            nq = fmaf(n[e], q, nq);
-        }
-        red[dg][j] = num;
-        if (j == 0) redn[dg] = nq;
-        __syncthreads();
-        if (dg == 0 && col < VD) {
-            const float nt = (red[0][j] + red[1][j]) + (red[2][j] + red[3][j]);
-            const float qt = (redn[0] + redn[1]) + (redn[2] + redn[3]);
-            a.o[(size_t)(start + t) * a.ld_o + (size_t)h * VD + col] = nt / (fmaxf(fabsf(qt), expf(-m)) + 1e-6f);
+            for (int e = 0; e < DPER; e++) {
+                const float kd = eb * sk[tt][d0 + e], q = sq[tt][d0 + e];
+                S[e] = fmaf(ea, S[e], kd * v);
+                n[e] = fmaf(ea, n[e], kd);
+                num = fmaf(S[e], q, num);
+                nq = fmaf(n[e], q, nq);
+            }
+            const int pb = tt & 1;                              // (two sets of partial sums: one barrier per token is enough)
+            red[pb][dg][j] = num;
+            if (j == 0) redn[pb][dg] = nq;
+            __syncthreads();
+            if (dg == 0 && col < VD) {
+                float nt = 0.0f, qt = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NDG; w++) { nt += red[pb][w][j]; qt += redn[pb][w]; }
+                a.o[(size_t)(start + t0 + tt) * a.ld_o + (size_t)h * VD + col] = nt / (fmaxf(fabsf(qt), expf(-m)) + 1e-6f);
+            }
         }
     }
 #pragma unroll
@@ -141,11 +137,13 @@ hipError_t launch_mlstm_scan(const MlstmArgs &a, hipStream_t st) {
     if (a.n_seg <= 0) return hipSuccess;
     if (!mlstm_shape_ok(a.D, a.VD)) return hipErrorInvalidValue;
     const dim3 grid((unsigned)a.n_seg, (unsigned)a.H, (unsigned)((a.VD + 63) / 64));
-    if (a.D <= 32) hipLaunchKernelGGL(mlstm_scan_kernel<8>, grid, dim3(256), 0, st, a);
-    else if (a.D <= 64) hipLaunchKernelGGL(mlstm_scan_kernel<16>, grid, dim3(256), 0, st, a);
-    else if (a.D <= 128) hipLaunchKernelGGL(mlstm_scan_kernel<32>, grid, dim3(256), 0, st, a);
-    else if (a.D <= 256) hipLaunchKernelGGL(mlstm_scan_kernel<64>, grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(mlstm_scan_kernel<128>, grid, dim3(256), 0, st, a);
+    // dim rows per thread x waves per workgroup: the waves of a workgroup split the rows of the state, the more of them the shorter a token's chain
+    if (a.D <= 16) hipLaunchKernelGGL((mlstm_scan_kernel<2, 8>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 32) hipLaunchKernelGGL((mlstm_scan_kernel<4, 8>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 64) hipLaunchKernelGGL((mlstm_scan_kernel<8, 8>), grid, dim3(512), 0, st, a);
+    else if (a.D <= 128) hipLaunchKernelGGL((mlstm_scan_kernel<8, 16>), grid, dim3(1024), 0, st, a);
+    else if (a.D <= 256) hipLaunchKernelGGL((mlstm_scan_kernel<16, 16>), grid, dim3(1024), 0, st, a);
+    else hipLaunchKernelGGL((mlstm_scan_kernel<32, 16>), grid, dim3(1024), 0, st, a);
     return hipGetLastError();
 }
 

@@ -209,23 +209,51 @@ __global__ __launch_bounds__(256) void mmb_mfma_kernel(MMBArgs a) {
         for (int j = 0; j < WT; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; if (GATED) acc2[i][j][r] = 0.0f; }
-    for (int k0 = 0; k0 < a.K; k0 += 16) {
-        bf16x8 wa[WT], wb[GATED ? WT : 1], xb[WT];
+    // PD steps of k are requested together, and the next PD while these are multiplied: a request per step in the chain would wait a memory round trip
+    // for every 16 of k.  Steps past K read the row's last step again and are never multiplied.
+    constexpr int PD = WT == 1 ? 4 : 2;
+    bf16x8 wa[2][PD][WT], wb[2][PD][GATED ? WT : 1];
+    f32x4 xa[2][PD][WT][2];
+    const int klast = a.K - 16;
+    const auto request = [&](int buf, int k0) {
 #pragma unroll
-        for (int i = 0; i < WT; i++) {
-            wa[i] = *reinterpret_cast<const bf16x8 *>(wr[i] + k0);
-            if (GATED) wb[i] = *reinterpret_cast<const bf16x8 *>(wr2[i] + k0);
-            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr[i] + k0), x1 = *reinterpret_cast<const f32x4 *>(xr[i] + k0 + 4);
-            u16x8 xb16 = {f2bf(x0.x), f2bf(x0.y), f2bf(x0.z), f2bf(x0.w), f2bf(x1.x), f2bf(x1.y), f2bf(x1.z), f2bf(x1.w)};
-            xb[i] = __builtin_bit_cast(bf16x8, xb16);
-        }
+        for (int u = 0; u < PD; u++) {
+            const int k = k0 + 16 * u <= klast ? k0 + 16 * u : klast;
 #pragma unroll
-        for (int i = 0; i < WT; i++)
-#pragma unroll
-            for (int j = 0; j < WT; j++) {
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[i], xb[j], acc[i][j], 0, 0, 0);
-                if (GATED) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[i], xb[j], acc2[i][j], 0, 0, 0);
+            for (int i = 0; i < WT; i++) {
+                wa[buf][u][i] = *reinterpret_cast<const bf16x8 *>(wr[i] + k);
+                if (GATED) wb[buf][u][i] = *reinterpret_cast<const bf16x8 *>(wr2[i] + k);
+                xa[buf][u][i][0] = *reinterpret_cast<const f32x4 *>(xr[i] + k);
+                xa[buf][u][i][1] = *reinterpret_cast<const f32x4 *>(xr[i] + k + 4);
             }
+        }
+    };
+    const auto multiply = [&](int buf, int k0) {
+#pragma unroll
+        for (int u = 0; u < PD; u++) {
+            if (k0 + 16 * u > klast) break;
+            bf16x8 xb[WT];
+#pragma unroll
+            for (int i = 0; i < WT; i++) {
+                const f32x4 x0 = xa[buf][u][i][0], x1 = xa[buf][u][i][1];
+                u16x8 xb16 = {f2bf(x0.x), f2bf(x0.y), f2bf(x0.z), f2bf(x0.w), f2bf(x1.x), f2bf(x1.y), f2bf(x1.z), f2bf(x1.w)};
+                xb[i] = __builtin_bit_cast(bf16x8, xb16);
+            }
+#pragma unroll
+            for (int i = 0; i < WT; i++)
+#pragma unroll
+                for (int j = 0; j < WT; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[buf][u][i], xb[j], acc[i][j], 0, 0, 0);
+                    if (GATED) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[buf][u][i], xb[j], acc2[i][j], 0, 0, 0);
+                }
+        }
+    };
+    request(0, 0);
+    for (int k0 = 0; k0 < a.K; k0 += 32 * PD) {
+        request(1, k0 + 16 * PD);
+        multiply(0, k0);
+        request(0, k0 + 32 * PD);
+        multiply(1, k0 + 16 * PD);
     }
     // register r of a lane: weight row (r & 3) + 8 (r >> 2) + 4 kg of the tile, token = lane & 31
 #pragma unroll

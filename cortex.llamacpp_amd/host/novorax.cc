@@ -329,8 +329,8 @@ bool Context::init_novorax(std::string &err) {
     d_tok_ = (int32_t *)(d_stage_ + 16);
     d_pos_ = d_tok_ + Tp; d_seq_ = d_pos_ + Tp; d_cell_ = d_seq_ + Tp; d_outrow_ = d_cell_ + Tp;
     d_seqmask_ = (uint64_t *)(d_outrow_ + Tp);
-    d_seg_ = (int32_t *)dalloc(3 * T * 4);
-    if (!d_seg_ || hipHostMalloc((void **)&h_seg_, 3 * T * 4, hipHostMallocDefault) != hipSuccess) { err = "segment list allocation failed"; return false; }
+    d_seg_ = (int32_t *)dalloc(4 * T * 4);
+    if (!d_seg_ || hipHostMalloc((void **)&h_seg_, 4 * T * 4, hipHostMallocDefault) != hipSuccess) { err = "segment list allocation failed"; return false; }
 
     // cache planes and recurrent state
     nvx_cache_.assign((size_t)M.n_latent_runs, nullptr);
@@ -365,6 +365,11 @@ bool Context::init_novorax(std::string &err) {
     nvx_att_ = (float *)dalloc(T * (size_t)std::max(M.max_att, 1) * 4);
     nvx_o_ = (float *)dalloc(T * (size_t)std::max(M.max_att, 1) * 4);
     nvx_ff_ = (float *)dalloc(T * TOP * (size_t)std::max(M.max_ff, 1) * 4);
+    {
+        int kr = 1;
+        for (const NvxLayer &L : M.layers) if (L.type == NVX_LATENT) kr = std::max(kr, L.kv_rank);
+        nvx_part_ = (float *)dalloc((size_t)LATENT_ATTN_SPLIT_MAX_PAIRS * LATENT_ATTN_SPLITS * (size_t)(kr + 2) * 4);
+    }
     if (!x_ || !xn_ || !xo_ || !nvx_x0_ || !nvx_xcat_ || !nvx_y_ || !nvx_a_ || !nvx_cq_ || !nvx_q_ || !nvx_qa_ || !nvx_lat_ || !nvx_att_ || !nvx_o_ || !nvx_ff_) { err = "activation buffer allocation failed"; return false; }
     if (M.max_top > 0) {
         nvx_xg_ = (float *)dalloc(T * TOP * W * 4);
@@ -416,8 +421,29 @@ void Context::nvx_state_copy(int src, int dst) {
     nvx_seq_len_[(size_t)dst] = nvx_seq_len_[(size_t)src];
 }
 
-bool Context::nvx_stage_segments(int n, const int32_t *seq) {
+bool Context::nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, const int *tcell) {
     const size_t T = cp.n_ubatch;
+    {
+        // per token: one past the highest cell its attention can need - the sequence's cells from earlier batches, and this batch's own cells up to the token
+        // (positions grow along a sequence's rows of a batch; a row that breaks that order falls back to the high-water mark)
+        int32_t *hi = h_seg_ + 3 * T;
+        int base[64], last_pos[64];
+        for (int s = 0; s < 64; s++) { base[s] = 0; last_pos[s] = -1; }
+        std::vector<char> mine(cells_.size(), 0);
+        for (int i = 0; i < n; i++) mine[(size_t)tcell[i]] = 1;
+        for (size_t c = 0; c < cells_.size(); c++) {
+            if (cells_[c].pos < 0 || mine[c]) continue;
+            uint64_t mk = cells_[c].seqs;
+            while (mk) { const int s = __builtin_ctzll(mk); mk &= mk - 1; base[s] = (int)c + 1; }
+        }
+        for (int i = 0; i < n; i++) {
+            const int s = seq[i] & 63;
+            if (pos[i] < last_pos[s]) base[s] = (int)cells_.size();
+            last_pos[s] = pos[i];
+            base[s] = std::max(base[s], tcell[i] + 1);
+            hi[i] = base[s];
+        }
+    }
     int32_t *start = h_seg_, *len = h_seg_ + T, *slot = h_seg_ + 2 * T;
     int ns = 0;
     for (int i = 0; i < n; i++) {
@@ -435,7 +461,7 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq) {
         seen |= bit;
     }
     if (ns > first) nvx_waves_.push_back({first, ns - first});
-    return hipMemcpyAsync(d_seg_, h_seg_, 3 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
+    return hipMemcpyAsync(d_seg_, h_seg_, 4 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
 }
 
 // pn != nullptr: the rows of x are RMS-normed with weight (1 + pn) on the way in (few rows: inside the launch; batches: a norm launch into xn_ first)
@@ -529,6 +555,8 @@ hipError_t Context::run_layers_novorax(int T) {
             aa.T = T; aa.H = H; aa.dim = L.dim; aa.rot = L.rot; aa.kv_rank = KR; aa.rot_dims = L.rot_dims; aa.cache = cache;
             aa.cell_pos = d_cell_pos_; aa.cell_seq = d_cell_seq_; aa.tok_pos = d_pos_; aa.tok_seq = d_seq_; aa.n_kv_dev = d_nkv_;
             aa.window = L.window; aa.scale = L.scale; aa.sink = L.sink; aa.rot_freq = L.rot_freq; aa.rot_mscale = L.rot_mscale;
+            aa.tok_hi = d_seg_ + 3 * (size_t)cp.n_ubatch;
+            if (nvx_part_ && (long long)T * H <= LATENT_ATTN_SPLIT_MAX_PAIRS) { aa.part = nvx_part_; aa.splits = LATENT_ATTN_SPLITS; }
             NVX_TRY(launch_latent_attn(aa, stream_));
             MMBArgs ua;                                         // att[t][h] = W_uv_h lat[t][h]
             ua.x = nvx_lat_; ua.ldx = H * KR; ua.x_zs = KR; ua.w = L.uv.w; ua.ldw = KR; ua.w_zs = (long long)L.vdim * KR;

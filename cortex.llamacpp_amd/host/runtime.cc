@@ -1934,7 +1934,7 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
     static const bool profiler_safe = getenv("MI355_PROFILER_SAFE") && getenv("MI355_PROFILER_SAFE")[0] == '1';
     if (profiler_safe) (void)hipStreamSynchronize(stream_);
     if (model->nvx) {
-        if (!nvx_stage_segments(n, seq)) { if (last_error.empty()) last_error = "segment list upload failed"; return -1; }
+        if (!nvx_stage_segments(n, seq, pos, tcell.data())) { if (last_error.empty()) last_error = "segment list upload failed"; return -1; }
         for (int i = 0; i < n; i++) nvx_seq_len_[(size_t)seq[i]] = std::max<uint64_t>(nvx_seq_len_[(size_t)seq[i]], (uint64_t)pos[i] + 1);
     }
     if (!stage_event_) (void)hipEventCreateWithFlags(&stage_event_, hipEventDisableTiming);

@@ -183,16 +183,18 @@ class Context {
     hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f,
                           const float *pn = nullptr);
     hipError_t nvx_feed_forward(const NvxLayer &L, int T);
-    bool nvx_stage_segments(int n, const int32_t *seq);     // runs of consecutive tokens of one sequence -> segment arrays (pinned, then device)
+    // runs of consecutive tokens of one sequence -> segment arrays; per-token scan bounds of the attention (pinned, then device)
+    bool nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, const int *tcell);
     void nvx_state_reset(int seq);                          // seq < 0: every slot
     void nvx_state_copy(int src, int dst);
     std::vector<float *> nvx_cache_;                        // [latent run] [n_ctx][kv_rank + rot]
     std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [mlstm run] [n_seq_max][H][D][VD], [..][H][D], [..][H]
     std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
     float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
+    float *nvx_part_ = nullptr;                             // split records of the latent attention of single-token steps
     float *nvx_att_ = nullptr, *nvx_o_ = nullptr, *nvx_ff_ = nullptr, *nvx_xg_ = nullptr, *nvx_yg_ = nullptr;
     int32_t *nvx_ids_ = nullptr, *nvx_meta_ = nullptr, *nvx_slot_ = nullptr, *nvx_tokof_ = nullptr;
-    int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [3][n_ubatch]: start, length, slot of every segment
+    int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [4][n_ubatch]: start, length, slot of every segment; scan bound of every token
     std::vector<std::pair<int, int>> nvx_waves_;            // segment ranges [first, count) that may share a launch (no slot twice)
     hipError_t run_output(int n_out, int out_base);
     hipError_t linear(const DevTensor &w, const ActQuant &aq, const float *x_f32, int K, int T, float *out, int ld_out,
