@@ -254,6 +254,10 @@ def test_a_token_far_back_stays_in_the_matrix_memory(pkg, tmp_path):
     ("big_recurrence", S.config([S.mlstm(heads=2, dim=144, vdim=200, mlp=S.dense(ff=264))], width=128, vocab=77)),
     ("no_rotation", S.config([S.latent(rot_dim=0, scaling=None, mlp=None)], width=64, vocab=40)),
     ("odd_width", S.config([S.latent(mlp=S.dense(ff=50)), S.mlstm(mlp=S.experts(ff=30))], width=50, vocab=33, loop=(1, 2, 2))),
+    # cache rows that are no multiple of 16 bytes (the attention kernel's scalar-load form), a state deeper than 256 rows, more experts than the grouped batch form takes
+    ("unaligned_latent", S.config([S.latent(heads=2, dim=10, rot_dim=6, vdim=14, kv_rank=37, q_rank=22, window=6, mlp=S.dense(ff=30))], width=44, vocab=29)),
+    ("deep_recurrence", S.config([S.mlstm(heads=1, dim=300, vdim=70, mlp=None)], width=64, vocab=41)),
+    ("many_experts", S.config([S.mlstm(heads=2, dim=8, vdim=8, mlp=S.experts(n=70, top=3, ff=16))], width=32, vocab=90)),
 ])
 def test_other_sizes(pkg, tmp_path, name, cfg):
     rig = Rig(pkg, tmp_path / name, cfg, seed=21)
