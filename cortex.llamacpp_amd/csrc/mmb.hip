@@ -55,6 +55,81 @@ __device__ __forceinline__ ZView z_view(const MMBArgs &a, int z) {
 }
 
 // ---------------------------------------------------------------- few rows: one wave per output column
+// Few rows against MANY output columns (single-token steps: the head, the feed-forward): a wave owns NR adjacent weight rows and keeps the activations of a
+// 512-wide piece of k in registers for all of them - the activation and norm-weight loads, which every wave repeats out of the caches, are paid once per NR
+// weight rows instead of once per row.  Up to TBR rows of X; 16-byte aligned operands; same arithmetic per output as mmb_vec_kernel.
+template <int NR, int TBR>
+__global__ __launch_bounds__(256) void mmb_vec_rows_kernel(MMBArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wave) * NR;
+    const ZView v = z_view(a, blockIdx.y);
+    if (n0 >= a.N) return;
+    const bool pn = a.pn_w != nullptr, gated = v.w2 != nullptr;
+    const unsigned short *wr[NR], *wr2[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const int n = n0 + r < a.N ? n0 + r : a.N - 1;          // rows past the end read the last row; their results are never stored
+        wr[r] = v.w + (size_t)n * a.ldw;
+        wr2[r] = gated ? v.w2 + (size_t)n * a.ldw : wr[r];
+    }
+    float acc[NR][TBR], acc2[NR][TBR], ss[TBR];
+#pragma unroll
+    for (int i = 0; i < TBR; i++) {
+        ss[i] = 0.0f;
+#pragma unroll
+        for (int r = 0; r < NR; r++) { acc[r][i] = 0.0f; acc2[r][i] = 0.0f; }
+    }
+    const int nt = v.rows < TBR ? v.rows : TBR;
+    for (int k = lane * 8; k < a.K; k += 512) {
+        u16x8 w8[NR], w28[NR];
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            w8[r] = *reinterpret_cast<const u16x8 *>(wr[r] + k);
+            if (gated) w28[r] = *reinterpret_cast<const u16x8 *>(wr2[r] + k);
+        }
+        float pw[8];
+        if (pn) {
+            const f32x4 g0 = *reinterpret_cast<const f32x4 *>(a.pn_w + k), g1 = *reinterpret_cast<const f32x4 *>(a.pn_w + k + 4);
+            pw[0] = a.pn_off + g0.x; pw[1] = a.pn_off + g0.y; pw[2] = a.pn_off + g0.z; pw[3] = a.pn_off + g0.w;
+            pw[4] = a.pn_off + g1.x; pw[5] = a.pn_off + g1.y; pw[6] = a.pn_off + g1.z; pw[7] = a.pn_off + g1.w;
+        }
+#pragma unroll
+        for (int i = 0; i < TBR; i++) {
+            if (i >= nt) break;
+            const float *xr = v.x + (size_t)i * a.ldx + k;
+            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xr), x1 = *reinterpret_cast<const f32x4 *>(xr + 4);
+            float xs[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            if (pn) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) { ss[i] = fmaf(xs[e], xs[e], ss[i]); xs[e] = xs[e] * pw[e]; }
+            }
+#pragma unroll
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    acc[r][i] = fmaf(xs[e], bf2f(w8[r][e]), acc[r][i]);
+                    if (gated) acc2[r][i] = fmaf(xs[e], bf2f(w28[r][e]), acc2[r][i]);
+                }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TBR; i++) {
+        if (i >= nt) break;
+        float q = ss[i];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+        const float inv = pn ? 1.0f / sqrtf(q / (float)a.K + a.pn_eps) : 1.0f;
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            float s1 = acc[r][i], s2 = acc2[r][i];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o, 64); s2 += __shfl_xor(s2, o, 64); }
+            if (pn) { s1 *= inv; s2 *= inv; }
+            if (lane == 0 && n0 + r < a.N) v.y[(size_t)i * a.ldy + n0 + r] = epi_apply(a.epi, s1, s2) * a.out_scale;
+        }
+    }
+}
+
 // With the norm prologue the row's sum of squares is gathered in the same pass as the products: y = inv_rms(x) * sum_k w_k (x_k (off + g_k)) - one trip
 // through memory per wave, the scale applied to the finished sum.
 template <bool VEC>
@@ -284,6 +359,13 @@ hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     if (a.pn_w && rows_max > MMB_VEC_ROWS) return hipErrorInvalidValue;   // (the norm prologue lives in the few-rows kernel only)
     if (rows_max <= MMB_VEC_ROWS || a.sel) {
         const dim3 grid((unsigned)((a.N + 3) / 4), (unsigned)a.nz);
+        // many columns, a handful of rows: four weight rows per wave (the grid still has thousands of waves)
+        if (vec && !a.sel && !a.meta && rows_max <= 4 && (long long)a.N * a.nz >= 4096) {
+            const dim3 g4((unsigned)((a.N + 15) / 16), (unsigned)a.nz);
+            if (rows_max == 1) hipLaunchKernelGGL((mmb_vec_rows_kernel<4, 1>), g4, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((mmb_vec_rows_kernel<4, 4>), g4, dim3(256), 0, st, a);
+            return hipGetLastError();
+        }
         if (vec) hipLaunchKernelGGL(mmb_vec_kernel<true>, grid, dim3(256), 0, st, a);
         else hipLaunchKernelGGL(mmb_vec_kernel<false>, grid, dim3(256), 0, st, a);
         return hipGetLastError();

@@ -267,6 +267,18 @@ def test_other_sizes(pkg, tmp_path, name, cfg):
     assert row_err(got, want) <= F32_TOL
 
 
+def test_wide_outputs_with_one_to_four_rows(pkg, tmp_path):
+    """Projections with thousands of output columns and one to four rows take the four-weight-rows-per-wave form of the weight-stream kernel (head,
+    feed-forward, the experts' pair products stay on the per-row form): portions of 1, 3 and 4 tokens in both precisions."""
+    cfg = S.config([S.latent(mlp=S.dense(ff=4104)), S.mlstm(mlp=S.experts(n=3, top=2, ff=48))], width=64, vocab=4099)
+    rig = Rig(pkg, tmp_path / "wide", cfg, seed=17)
+    t = toks(26, cfg["vocab"], 19)
+    want = rig.ref(t)
+    for exact, tol in ((True, F32_TOL), (False, F32_TOL)):     # (up to 16 rows the activations stay f32 in either precision)
+        got = feed_in_portions(rig.ctx(exact=exact), t, [1, 3, 4, 2])
+        assert row_err(got, want) <= tol, exact
+
+
 # ------------------------------------------------------------------------------------------ serving precision, graphs
 def row_errs(got, want):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
