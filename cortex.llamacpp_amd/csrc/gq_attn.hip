@@ -1,0 +1,265 @@
+// gq_attn.hip — grouped-query attention with a sliding window on f32 cache rows, for the bf16-weight models.
+//
+// A token's cache row is [k_0 .. k_{G-1} | v_0 .. v_{G-1}]: G key heads of dim floats, then G value heads of vdim floats; query head h reads key / value
+// head h / (H / G).  Visibility: same sequence, 0 <= pos_query - pos_cell < window (window 0: every earlier cell).  Plain softmax over the visible cells; an
+// optional per-head sink logit joins the denominator; an optional output gate multiplies head h's result by sigmoid(gate[t][h]).  Everything here is f32:
+// positions, angles, norms, scores, weights, the running sums.
+//
+// gq_prep: per token, behind the fused q | k | v projection: an optional RMS norm over the WHOLE query projection (all heads at once) and over the whole key
+// projection, with plain weights; the rotation of the first rot_dims entries of every query and key head in the rotate-half layout (entry i pairs with entry
+// i + rot_dims / 2; the per-pair angle table comes from the host); the score multipliers (one number for the layer, one per head) folded into the query;
+// keys and values stored to the token's cache row.
+#include "kernels.h"
+
+namespace mi355 {
+
+namespace {
+
+__device__ __forceinline__ float gq_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ float gq_block_sum_256(float v, float *sh) {
+    v = gq_wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+
+__global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
+    __shared__ float sh[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int NQ = a.H * a.dim, NK = a.G * a.dim, NV = a.G * a.vdim, half = a.rot_dims >> 1;
+    const float *qr = a.p + (size_t)t * a.ld_p, *kr = qr + NQ, *vr = kr + NK;
+    float inv_q = 1.0f, inv_k = 1.0f;
+    if (a.wq_norm) {
+        float ss = 0.0f;
+        for (int i = tid; i < NQ; i += 256) { const float v = qr[i]; ss = fmaf(v, v, ss); }
+        inv_q = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NQ + a.eps);
+    }
+    if (a.wk_norm) {
+        float ss = 0.0f;
+        for (int i = tid; i < NK; i += 256) { const float v = kr[i]; ss = fmaf(v, v, ss); }
+        inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
+    }
+    const float p = (float)a.tok_pos[t];
+    float *qo = a.q + (size_t)t * a.ld_q;
+    float *row = a.cache + (size_t)a.tok_cell[t] * (size_t)(NK + NV);
+    // one loop over the query entries, then the key entries: element (head, d) of either
+    for (int i = tid; i < NQ + NK; i += 256) {
+        const bool isq = i < NQ;
+        const int e = isq ? i : i - NQ, d = e % a.dim, b = e - d;
+        const float *src = isq ? qr : kr;
+        const float *wn = isq ? a.wq_norm : a.wk_norm;
+        const float inv = isq ? inv_q : inv_k;
+        float o;
+        if (d < a.rot_dims) {
+            const int j = d < half ? d : d - half;
+            const float ang = p * a.rot_freq[j], c = cosf(ang), s = sinf(ang);
+            float u = src[b + j] * inv, w = src[b + j + half] * inv;
+            if (wn) { u *= wn[b + j]; w *= wn[b + j + half]; }
+            o = d < half ? u * c - w * s : w * c + u * s;
+        } else {
+            o = src[e] * inv;
+            if (wn) o *= wn[e];
+        }
+        if (isq) {
+            float m = a.q_scale;
+            if (a.head_scale) m *= a.head_scale[e / a.dim];
+            qo[e] = o * m;
+        } else row[e] = o;
+    }
+    for (int i = tid; i < NV; i += 256) row[NK + i] = vr[i];
+}
+
+constexpr int GQ_MAX_D = 256;                                   // dim and vdim the attention kernel is instantiated for (4 x 64)
+
+// One workgroup per (token, head), NW waves.  A wave works on four cells at a time: each 16-lane group owns one cell, its lanes hold elements
+// 64 j + 4 li .. + 3 of the key head and of the value head (16-byte loads) and the matching running sums; the next four cells of the wave are requested
+// before the current ones are used.  Every group keeps its own running maximum / sum / weighted value; groups, then waves, are merged at the end together
+// with the sink term and the output gate.  NJ = ceil(max(dim, vdim) / 64); VEC: key and value heads start on 16-byte boundaries.
+template <int NJ, bool VEC>
+__global__ __launch_bounds__(512) void gq_attn_kernel(GqAttnArgs a) {
+    extern __shared__ float lds[];
+    const int D = a.dim, VD = a.vdim, LP = NJ * 64;
+    const int NW = blockDim.x >> 6;
+    float *qv = lds;                                            // [LP] (zero beyond dim)
+    float *wm = lds + LP, *wl = wm + NW, *wacc = wl + NW;        // [NW], [NW], [NW][LP]
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, li = lane & 15;
+    const int kvh = h / (a.H / a.G);
+    const size_t L = (size_t)a.G * (D + VD), koff = (size_t)kvh * D, voff = (size_t)a.G * D + (size_t)kvh * VD;
+    const int tpos = a.tok_pos[t];
+    const uint64_t sbit = 1ull << (a.tok_seq[t] & 63);
+    for (int i = tid; i < LP; i += blockDim.x) qv[i] = i < D ? a.q[(size_t)t * a.ld_q + (size_t)h * D + i] : 0.0f;
+    __syncthreads();
+    float acc[NJ][4], ck[NJ][4], cv[NJ][4], nk[NJ][4], nv[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) { acc[j][e] = 0.0f; ck[j][e] = 0.0f; cv[j][e] = 0.0f; nk[j][e] = 0.0f; nv[j][e] = 0.0f; }
+    float m = -INFINITY, l = 0.0f;
+    int n_kv = *a.n_kv_dev;
+    if (a.tok_hi) n_kv = a.tok_hi[t] < n_kv ? a.tok_hi[t] : n_kv;
+    const int stride = NW * 4;
+    // the scanned cells: [first cell that can still be inside the token's window, one past the token's own cells); gridDim.z > 1 (steps of a few tokens)
+    // cuts them into that many runs, one workgroup each, whose records gq_attn_merge_kernel joins
+    int c_lo = a.tok_lo ? a.tok_lo[t] : 0, c_hi = n_kv;
+    if (c_lo > c_hi) c_lo = c_hi;
+    if (gridDim.z > 1) {
+        const int per = ((c_hi - c_lo + (int)gridDim.z - 1) / (int)gridDim.z + stride - 1) / stride * stride;
+        c_lo += (int)blockIdx.z * per;
+        c_hi = c_lo + per < c_hi ? c_lo + per : c_hi;
+    }
+    const auto visible = [&](int c) {
+        if (c >= c_hi) return false;
+        const int cp = a.cell_pos[c];
+        return cp >= 0 && cp <= tpos && (a.cell_seq[c] & sbit) != 0 && !(a.window > 0 && tpos - cp >= a.window);
+    };
+    const auto fetch = [&](int c, bool vis, float (&dk)[NJ][4], float (&dv)[NJ][4]) {
+        const float *kr = a.cache + (size_t)c * L + koff, *vr = a.cache + (size_t)c * L + voff;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const int e0 = 64 * j + 4 * li;
+            if (VEC) {
+                float4 k4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), v4 = k4;
+                if (vis && e0 < D) k4 = *reinterpret_cast<const float4 *>(kr + e0);
+                if (vis && e0 < VD) v4 = *reinterpret_cast<const float4 *>(vr + e0);
+                dk[j][0] = k4.x; dk[j][1] = k4.y; dk[j][2] = k4.z; dk[j][3] = k4.w;
+                dv[j][0] = v4.x; dv[j][1] = v4.y; dv[j][2] = v4.z; dv[j][3] = v4.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    dk[j][e] = vis && e0 + e < D ? kr[e0 + e] : 0.0f;
+                    dv[j][e] = vis && e0 + e < VD ? vr[e0 + e] : 0.0f;
+                }
+            }
+        }
+    };
+    int c = c_lo + wave * 4 + g;
+    bool vis = visible(c);
+    fetch(c, vis, ck, cv);
+    for (int c0 = c_lo; c0 < c_hi; c0 += stride) {              // (uniform trip count: the shuffles below are executed by whole waves)
+        const int cn = c + stride;
+        const bool visn = visible(cn);
+        fetch(cn, visn, nk, nv);
+        float dot = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const float4 q4 = *reinterpret_cast<const float4 *>(qv + 64 * j + 4 * li);
+            dot = fmaf(ck[j][0], q4.x, dot); dot = fmaf(ck[j][1], q4.y, dot); dot = fmaf(ck[j][2], q4.z, dot); dot = fmaf(ck[j][3], q4.w, dot);
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+        if (vis) {
+            const float mn = fmaxf(m, dot), alpha = expf(m - mn), p = expf(dot - mn);   // (m = -inf at the group's first cell: alpha = 0)
+            l = l * alpha + p;
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[j][e] = acc[j][e] * alpha + p * cv[j][e];
+            m = mn;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) { ck[j][e] = nk[j][e]; cv[j][e] = nv[j][e]; }
+        c = cn; vis = visn;
+    }
+    // the four groups of a wave -> one record per wave
+    float M = fmaxf(m, __shfl_xor(m, 16, 64));
+    M = fmaxf(M, __shfl_xor(M, 32, 64));
+    const float sg = l > 0.0f ? expf(m - M) : 0.0f;
+    l *= sg;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float v = acc[j][e] * sg;
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            if (g == 0) wacc[wave * LP + 64 * j + 4 * li + e] = v;
+        }
+    if (lane == 0) { wm[wave] = M; wl[wave] = l; }
+    __syncthreads();
+    if (gridDim.z > 1) {                                        // this run's record: maximum, sum, weighted value (sink and gate enter at the merge)
+        float *rec = a.part + (((size_t)t * a.H + h) * gridDim.z + blockIdx.z) * (size_t)(VD + 2);
+        float Ms = -INFINITY;
+        for (int w = 0; w < NW; w++) if (wl[w] > 0.0f) Ms = fmaxf(Ms, wm[w]);
+        float ls = 0.0f;
+        for (int w = 0; w < NW; w++) ls += wl[w] > 0.0f ? wl[w] * expf(wm[w] - Ms) : 0.0f;
+        if (tid == 0) { rec[0] = Ms; rec[1] = ls; }
+        for (int i = tid; i < VD; i += blockDim.x) {
+            float o = 0.0f;
+            for (int w = 0; w < NW; w++) o += wl[w] > 0.0f ? wacc[w * LP + i] * expf(wm[w] - Ms) : 0.0f;
+            rec[2 + i] = o;
+        }
+        return;
+    }
+    float MM = a.sink ? a.sink[h] : -INFINITY;
+    for (int w = 0; w < NW; w++) if (wl[w] > 0.0f) MM = fmaxf(MM, wm[w]);
+    float den = a.sink ? expf(a.sink[h] - MM) : 0.0f;
+    for (int w = 0; w < NW; w++) den += wl[w] > 0.0f ? wl[w] * expf(wm[w] - MM) : 0.0f;
+    float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
+    for (int i = tid; i < VD; i += blockDim.x) {
+        float o = 0.0f;
+        for (int w = 0; w < NW; w++) o += wl[w] > 0.0f ? wacc[w * LP + i] * expf(wm[w] - MM) : 0.0f;
+        a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
+    }
+}
+
+__global__ __launch_bounds__(256) void gq_attn_merge_kernel(GqAttnArgs a, int splits) {
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, VD = a.vdim;
+    const float *rec = a.part + ((size_t)t * a.H + h) * splits * (size_t)(VD + 2);
+    float MM = a.sink ? a.sink[h] : -INFINITY;
+    for (int s = 0; s < splits; s++) if (rec[(size_t)s * (VD + 2) + 1] > 0.0f) MM = fmaxf(MM, rec[(size_t)s * (VD + 2)]);
+    float den = a.sink ? expf(a.sink[h] - MM) : 0.0f;
+    for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (VD + 2); den += r[1] > 0.0f ? r[1] * expf(r[0] - MM) : 0.0f; }
+    float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)t * a.ld_gate + h]));
+    for (int i = tid; i < VD; i += 256) {
+        float o = 0.0f;
+        for (int s = 0; s < splits; s++) { const float *r = rec + (size_t)s * (VD + 2); o += r[1] > 0.0f ? r[2 + i] * expf(r[0] - MM) : 0.0f; }
+        a.out[(size_t)t * a.ld_out + (size_t)h * VD + i] = o * inv;
+    }
+}
+
+template <int NJ>
+static hipError_t launch_gq_attn_nj(const GqAttnArgs &a, hipStream_t st) {
+    // few (token, head) pairs - steps of a few tokens - get eight waves each: more cells in flight where the grid alone cannot fill the device
+    const int nw = (long long)a.T * a.H <= 1024 ? 8 : 4;
+    const size_t lds = (size_t)(NJ * 64 + 2 * nw + nw * NJ * 64) * sizeof(float);
+    const bool vec = (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0;
+    const int splits = a.part && a.splits > 1 ? a.splits : 1;
+    const dim3 grid((unsigned)a.T, (unsigned)a.H, (unsigned)splits);
+    if (vec) hipLaunchKernelGGL((gq_attn_kernel<NJ, true>), grid, dim3(64 * nw), lds, st, a);
+    else hipLaunchKernelGGL((gq_attn_kernel<NJ, false>), grid, dim3(64 * nw), lds, st, a);
+    if (splits > 1) hipLaunchKernelGGL(gq_attn_merge_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a, splits);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool gq_attn_shape_ok(int H, int G, int dim, int vdim) { return H >= 1 && G >= 1 && H % G == 0 && dim >= 1 && vdim >= 1 && dim <= GQ_MAX_D && vdim <= GQ_MAX_D; }
+
+hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
+    if (a.T <= 0) return hipSuccess;
+    if (a.rot_dims < 0 || a.rot_dims > a.dim || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
+    if (a.T <= 0) return hipSuccess;
+    if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim)) return hipErrorInvalidValue;
+    const int Dm = a.dim > a.vdim ? a.dim : a.vdim;
+    if (Dm <= 64) return launch_gq_attn_nj<1>(a, st);
+    if (Dm <= 128) return launch_gq_attn_nj<2>(a, st);
+    return launch_gq_attn_nj<4>(a, st);
+}
+
+}  // namespace mi355

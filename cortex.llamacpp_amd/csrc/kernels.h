@@ -285,6 +285,45 @@ hipError_t launch_add_row(float *x, const float *row, int n, int T, hipStream_t 
 hipError_t launch_moe_table_ids(const int32_t *table, const int32_t *tok, int T, int k, int32_t *ids, hipStream_t st);   // ids[t][j] = table[tok[t]][j]
 hipError_t launch_moe_uniform_combine(float *out, const float *y, const int32_t *slot_of, int T, int E, int k, float w, hipStream_t st);
 
+// router with expert groups (misc.hip): s = softmax(z[t][0 .. E)) (row stride ld_z); the experts form n_group equal groups of neighbours, a group scores as its
+// largest s, only experts of the `keep` best groups can be taken; the k best of them, weights s / (their sum + 1e-20) * scale.  ids / w: [T][k], best first.
+constexpr int MOE_ROUTE_MAX_EXPERTS = 8192;
+hipError_t launch_moe_route_groups(const float *z, int ld_z, int T, int E, int k, int n_group, int keep, float scale, int32_t *ids, float *w, hipStream_t st);
+// x[t][:] += m * (a[t] + b[t] + sum_j w[t][j] * y[row(t, j)]): the close of a block whose mixer (a), always-on expert (b, nullable) and routed experts (y; k = 0:
+// none) all read the same normed input; row(t, j) = slot_of[t * k + j], or t * k + j without a grouping
+hipError_t launch_block_combine(float *x, const float *a, const float *b, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, float m, hipStream_t st);
+
+// ---------------------------------------------------------------- grouped-query attention on f32 cache rows (gq_attn.hip)
+// cache row of a cell: [G key heads of dim | G value heads of vdim] f32.  Query head h reads key / value head h / (H / G).
+struct GqPrepArgs {
+    const float *p; int ld_p;              // [T][q: H*dim | k: G*dim | v: G*vdim | ...] projections of the batch
+    int T, H, G, dim, vdim;
+    const float *wq_norm, *wk_norm; float eps;   // nullable: RMS norm over the whole query / key projection (all heads at once), plain weights [H*dim] / [G*dim]
+    int rot_dims; const float *rot_freq;   // the first rot_dims entries of every q / k head turn, entry i with entry i + rot_dims / 2; [rot_dims / 2] radians per position
+    float q_scale; const float *head_scale;      // the query is multiplied by q_scale * head_scale[h] (nullable): the score's constant factors
+    const int32_t *tok_pos, *tok_cell;
+    float *q; int ld_q;                    // [T][H*dim]: normed, turned, scaled queries
+    float *cache;                          // [n_ctx][G*dim + G*vdim]
+};
+hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st);
+struct GqAttnArgs {
+    const float *q; int ld_q;              // [T][H][dim] from launch_gq_prep
+    float *out; int ld_out;                // [T][H][vdim]
+    int T, H, G, dim, vdim;
+    const float *cache;
+    const int32_t *cell_pos; const uint64_t *cell_seq; const int32_t *tok_pos, *tok_seq; const int32_t *n_kv_dev;
+    int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
+    const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
+    const float *gate; int ld_gate;        // nullable: head h's output is multiplied by sigmoid(gate[t * ld_gate + h])
+    // steps of a few tokens: the scanned cells cut into `splits` runs, one workgroup each, merged afterwards; part: T * H * splits * (vdim + 2) floats
+    float *part; int splits;
+    // nullable, per token, host-made from the cell table: one past the highest cell that can hold a key of its sequence at or before its position, and the
+    // lowest cell that can hold one still inside the window
+    const int32_t *tok_hi, *tok_lo;
+};
+bool gq_attn_shape_ok(int H, int G, int dim, int vdim);
+hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st);
+
 // ---------------------------------------------------------------- latent attention (latent_attn.hip)
 // cache row of a cell: [kv_rank normed latent | rot rotated shared key part] f32.  rot_freq: [rot_dims / 2] angles per position (host-made, YaRN blend
 // included), rot_mscale multiplies cos and sin; interleaved pairs over the first rot_dims entries of the rotated part.

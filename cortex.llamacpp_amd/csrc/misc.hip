@@ -539,6 +539,99 @@ hipError_t launch_moe_scatter_combine(float *x, const float *y, const float *w, 
     return hipGetLastError();
 }
 
+// Router of a mixture of experts whose experts form groups.  One wave per token: s = softmax(z) over all E experts (kept in LDS); a group is n / n_group
+// neighbouring experts and scores as its largest s; the `keep` best groups stay open (lowest index wins a tie); the k open experts with the largest s are
+// taken, best first; weights s / (sum of the taken + 1e-20) * scale.  n_group 1 (or keep >= n_group): plain top-k of the softmax.
+__global__ __launch_bounds__(64) void moe_route_groups_kernel(const float *z, int ld_z, int E, int k, int n_group, int keep, float scale, int32_t *ids, float *w) {
+    extern __shared__ float rl[];
+    float *s = rl, *gs = rl + E, *tw = gs + n_group;            // [E] scores (a taken expert's becomes -1), [n_group] group scores (an OPEN group's becomes -1), [k] taken scores
+    int *ti = reinterpret_cast<int *>(tw + k);                  // [k] taken experts
+    const int t = blockIdx.x, lane = threadIdx.x, per = E / n_group;
+    const float *zr = z + (size_t)t * ld_z;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) { const float p = expf(zr[e] - mx); s[e] = p; sum += p; }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    __syncthreads();
+    for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
+    __syncthreads();
+    // index of the largest v[i] >= 0 whose group is open (open_of == nullptr: every group), lowest index first; n when there is none
+    const auto arg_best = [&](const float *v, int n, const float *open_of, float &best) {
+        float bv = -1.0f; int bi = n;
+        for (int i = lane; i < n; i += 64) {
+            const float x = (open_of && open_of[i / per] >= 0.0f) ? -1.0f : v[i];
+            if (x > bv) { bv = x; bi = i; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64); const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        best = bv;
+        return bi;
+    };
+    const bool grouped = n_group > 1 && keep < n_group;
+    if (grouped) {
+        for (int gi = lane; gi < n_group; gi += 64) {
+            float gm = 0.0f;
+            for (int e = gi * per; e < (gi + 1) * per; e++) gm = fmaxf(gm, s[e]);
+            gs[gi] = gm;
+        }
+        __syncthreads();
+        for (int r = 0; r < keep; r++) {
+            float bv;
+            const int gi = arg_best(gs, n_group, nullptr, bv);
+            __syncthreads();
+            if (lane == 0 && gi < n_group) gs[gi] = -1.0f;
+            __syncthreads();
+        }
+    }
+    float tot = 0.0f;
+    for (int r = 0; r < k; r++) {
+        float bv;
+        int ei = arg_best(s, E, grouped ? gs : nullptr, bv);
+        if (ei >= E) { ei = 0; bv = 0.0f; }                      // (fewer open experts than k: refused by the launcher)
+        __syncthreads();
+        if (lane == 0) { ti[r] = ei; tw[r] = bv; s[ei] = -1.0f; }
+        tot += bv;
+        __syncthreads();
+    }
+    const float inv = scale / (tot + 1e-20f);
+    for (int r = lane; r < k; r += 64) { ids[(size_t)t * k + r] = ti[r]; w[(size_t)t * k + r] = tw[r] * inv; }
+}
+hipError_t launch_moe_route_groups(const float *z, int ld_z, int T, int E, int k, int n_group, int keep, float scale, int32_t *ids, float *w, hipStream_t st) {
+    if (T <= 0) return hipSuccess;
+    if (E < 1 || k < 1 || k > E || n_group < 1 || E % n_group != 0 || keep < 1 || E > MOE_ROUTE_MAX_EXPERTS) return hipErrorInvalidValue;
+    if (keep > n_group) keep = n_group;
+    if ((long long)keep * (E / n_group) < k) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(moe_route_groups_kernel, dim3((unsigned)T), dim3(64), (size_t)(E + n_group + 2 * k) * sizeof(float), st, z, ld_z, E, k, n_group, keep, scale, ids, w);
+    return hipGetLastError();
+}
+
+// The close of a block whose sublayers all read one normed input: x[t][d] += m * (a[t][d] + b[t][d] + sum_j w[t][j] * y[row(t, j)][d]); a = the mixer's output,
+// b = an always-on expert's (nullable), y = the routed experts' rows (row(t, j) = slot_of[t * k + j], or t * k + j without a grouping; k = 0: none), added in
+// rank order.
+__global__ void block_combine_kernel(float *x, const float *a, const float *b, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, float m) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)T * E) return;
+    const int t = (int)(i / E), d = (int)(i - (int64_t)t * E);
+    float o = 0.0f;
+    for (int j = 0; j < k; j++) o += y[(size_t)(slot_of ? slot_of[(size_t)t * k + j] : t * k + j) * E + d] * w[(size_t)t * k + j];
+    if (b) o += b[i];
+    if (a) o += a[i];
+    x[i] = x[i] + m * o;
+}
+hipError_t launch_block_combine(float *x, const float *a, const float *b, const float *y, const float *w, const int32_t *slot_of, int T, int E, int k, float m, hipStream_t st) {
+    if ((int64_t)T * E <= 0) return hipSuccess;
+    if (k > 0 && (!y || !w)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(block_combine_kernel, dim3((unsigned)(((int64_t)T * E + 255) / 256)), dim3(256), 0, st, x, a, b, y, w, slot_of, T, E, k, m);
+    return hipGetLastError();
+}
+
 __global__ void gather_rows_kernel(const float *src, const int32_t *rows, int n, float *dst) {
     const int r = blockIdx.y;
     const float *s = src + (size_t)rows[r] * n;

@@ -11,9 +11,7 @@
 #include <fstream>
 #include <sstream>
 
-#include "json.h"
-#include "runtime.h"
-#include "safetensors.h"
+#include "config_model.h"
 
 namespace mi355 {
 
@@ -28,7 +26,7 @@ void set_error(const char *fmt, ...);
         }                                                                                          \
     } while (0)
 
-bool novorax_path(const std::string &path, std::string &dir) {
+bool config_model_path(const std::string &path, std::string &dir) {
     struct stat st;
     if (stat(path.c_str(), &st) != 0) return false;
     dir = path;
@@ -41,71 +39,12 @@ bool novorax_path(const std::string &path, std::string &dir) {
     return stat((dir + "/config.json").c_str(), &st) == 0 && stat((dir + "/model.safetensors").c_str(), &st) == 0;
 }
 
-namespace {
-
-struct Loader {
-    SafeTensorsFile st;
-    Model *m = nullptr;
-    std::string err;
-    uint64_t bytes = 0;
-
-    void *dev(const void *host, size_t n) {
-        if (!err.empty()) return nullptr;
-        void *p = nullptr;
-        if (hipMalloc(&p, n ? n : 16) != hipSuccess) { err = "device allocation of " + std::to_string(n) + " bytes failed"; return nullptr; }
-        m->arenas.push_back((uint8_t *)p);
-        if (n && hipMemcpy(p, host, n, hipMemcpyHostToDevice) != hipSuccess) { err = "upload failed"; return nullptr; }
-        bytes += n;
-        return p;
-    }
-    const SafeTensor *need(const std::string &name, const char *dtype, std::initializer_list<int64_t> shape) {
-        if (!err.empty()) return nullptr;
-        const SafeTensor *t = st.find(name);
-        if (!t) { err = "tensor '" + name + "' missing"; return nullptr; }
-        if (t->dtype != dtype) { err = "tensor '" + name + "' is " + t->dtype + ", expected " + dtype; return nullptr; }
-        if (t->shape.size() != shape.size() || !std::equal(shape.begin(), shape.end(), t->shape.begin())) {
-            std::string want, have;
-            for (int64_t d : shape) want += (want.empty() ? "" : ", ") + std::to_string(d);
-            for (int64_t d : t->shape) have += (have.empty() ? "" : ", ") + std::to_string(d);
-            err = "tensor '" + name + "' has shape [" + have + "], the configuration asks for [" + want + "]";
-            return nullptr;
-        }
-        return t;
-    }
-    // several [rows_i][K] bf16 tensors under each other as one device matrix
-    BfMat rows(const std::vector<std::pair<std::string, int>> &parts, int K) {
-        BfMat o;
-        std::vector<unsigned short> host;
-        for (const auto &pr : parts) {
-            const SafeTensor *t = need(pr.first, "BF16", {pr.second, K});
-            if (!t) return o;
-            const unsigned short *s = (const unsigned short *)t->data;
-            host.insert(host.end(), s, s + (size_t)pr.second * K);
-            o.N += pr.second;
-        }
-        o.K = K;
-        o.w = (unsigned short *)dev(host.data(), host.size() * 2);
-        return o;
-    }
-    float *vec(const std::string &name, int n) {
-        const SafeTensor *t = need(name, "BF16", {n});
-        if (!t) return nullptr;
-        std::vector<float> h((size_t)n);
-        const unsigned short *s = (const unsigned short *)t->data;
-        for (int i = 0; i < n; i++) { const uint32_t u = (uint32_t)s[i] << 16; memcpy(&h[(size_t)i], &u, 4); }
-        return (float *)dev(h.data(), h.size() * 4);
-    }
-};
-
-bool positive(std::string &err, const char *what, int64_t v, int64_t hi = 1 << 24) {
-    if (v >= 1 && v <= hi) return true;
-    err = std::string("configuration: ") + what + " = " + std::to_string(v) + " is out of range";
-    return false;
-}
-
-}  // namespace
-
-Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int &status) {
+// the model registry of the folder models: configuration "architecture" -> the design's loader
+Model *config_model_load(const std::string &dir, int main_gpu, std::string &err, int &status) {
+    static const struct { const char *architecture; Model *(*build)(const Json &, const std::string &, Bf16Loader &, std::string &, int &); } designs[] = {
+        {"Novorax", novorax_build},
+        {"Fidepel", fidepel_build},
+    };
     status = -102;
     std::ifstream cf(dir + "/config.json");
     if (!cf) { err = "cannot open " + dir + "/config.json"; status = -101; return nullptr; }
@@ -114,19 +53,38 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
     Json cfg;
     std::string jerr;
     if (!Json::parse(ss.str(), cfg, &jerr) || !cfg.is_object()) { err = "config.json: " + jerr; return nullptr; }
-    if (cfg["architecture"].as_string() != "Novorax") { err = "config.json: unsupported architecture '" + cfg["architecture"].as_string() + "'"; return nullptr; }
-    std::unique_ptr<Model> m(new Model());
-    m->path = dir;
-    m->device = main_gpu;
-    if (hipSetDevice(main_gpu) != hipSuccess) { err = "hipSetDevice failed"; status = -103; return nullptr; }
-    Loader ld;
-    ld.m = m.get();
-    err = ld.st.open(dir + "/model.safetensors");
-    if (!err.empty()) { status = err.rfind("cannot", 0) == 0 ? -101 : -102; return nullptr; }
-    m->nvx.reset(new NovoraxModel());
+    const std::string arch = cfg["architecture"].as_string();
+    for (const auto &d : designs) {
+        if (arch != d.architecture) continue;
+        std::unique_ptr<Model> m(new Model());
+        m->path = dir;
+        m->device = main_gpu;
+        if (hipSetDevice(main_gpu) != hipSuccess) { err = "hipSetDevice failed"; status = -103; return nullptr; }
+        Bf16Loader ld;
+        ld.m = m.get();
+        err = ld.st.open(dir + "/model.safetensors");
+        if (!err.empty()) { status = err.rfind("cannot", 0) == 0 ? -101 : -102; return nullptr; }
+        m->nvx.reset(new NovoraxModel());
+        if (!d.build(cfg, dir, ld, err, status)) return nullptr;   // (m frees what was uploaded)
+        if (hipDeviceSynchronize() != hipSuccess) { err = "device synchronise failed behind the upload"; status = -103; return nullptr; }
+        m->device_bytes = ld.bytes;
+        m->file_tensor_bytes = ld.st.file_bytes();
+        if (!m->bytes_per_token) m->bytes_per_token = ld.bytes;
+        status = 0;
+        return m.release();
+    }
+    err = "config.json: unsupported architecture '" + arch + "'";
+    return nullptr;
+}
+
+Model *novorax_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, std::string &err, int &status) {
+    (void)dir;
+    status = -102;
+    Model *const m = ld.m;
     NovoraxModel &M = *m->nvx;
+    M.design = "novorax";
     const int W = (int)cfg["width"].as_int(), V = (int)cfg["vocab"].as_int();
-    if (!positive(err, "width", W) || !positive(err, "vocab", V)) return nullptr;
+    if (!cfg_positive(err, "width", W) || !cfg_positive(err, "vocab", V)) return nullptr;
     M.width = W; M.n_vocab = V;
     M.eps = (float)cfg["norm"]["eps"].as_double(1e-5);
     M.logit_scale = (float)cfg["logit_scale"].as_double(1.0);
@@ -134,17 +92,7 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
     if (!layers.is_array() || layers.size() == 0 || layers.size() > 1024) { err = "configuration: 'layers' must list 1 .. 1024 layers"; return nullptr; }
     const int nl = (int)layers.size();
 
-    // the embedding table keeps the row stride launch_get_rows expects
-    {
-        const SafeTensor *t = ld.need("embed", "BF16", {V, W});
-        if (t) {
-            const size_t rb = dev_row_bytes(T_BF16, W);
-            std::vector<uint8_t> host((size_t)V * rb, 0);
-            for (int r = 0; r < V; r++) memcpy(host.data() + (size_t)r * rb, t->data + (size_t)r * W * 2, (size_t)W * 2);
-            M.embed.w = (unsigned short *)ld.dev(host.data(), host.size());
-            M.embed.N = V; M.embed.K = W;
-        }
-    }
+    M.embed = ld.embedding("embed", V, W);
     M.head = ld.rows({{"head", V}}, W);
     M.final_norm = ld.vec("final.norm", W);
 
@@ -157,12 +105,12 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
         L.norm1 = ld.vec(p + "norm1", W);
         L.norm1b = ld.vec(p + "norm1b", W);
         L.heads = (int)mx["heads"].as_int(); L.dim = (int)mx["dim"].as_int(); L.vdim = (int)mx["vdim"].as_int();
-        if (!positive(err, "mixer.heads", L.heads, 4096) || !positive(err, "mixer.dim", L.dim, 1 << 16) || !positive(err, "mixer.vdim", L.vdim, 1 << 16)) return nullptr;
+        if (!cfg_positive(err, "mixer.heads", L.heads, 4096) || !cfg_positive(err, "mixer.dim", L.dim, 1 << 16) || !cfg_positive(err, "mixer.vdim", L.vdim, 1 << 16)) return nullptr;
         const int H = L.heads;
         if (type == "latent_attention") {
             L.type = NVX_LATENT;
             L.rot = (int)mx["rot_dim"].as_int(0); L.kv_rank = (int)mx["kv_rank"].as_int(); L.q_rank = (int)mx["q_rank"].as_int();
-            if (!positive(err, "mixer.kv_rank", L.kv_rank) || !positive(err, "mixer.q_rank", L.q_rank) || L.rot < 0) { if (err.empty()) err = "configuration: mixer.rot_dim is negative"; return nullptr; }
+            if (!cfg_positive(err, "mixer.kv_rank", L.kv_rank) || !cfg_positive(err, "mixer.q_rank", L.q_rank) || L.rot < 0) { if (err.empty()) err = "configuration: mixer.rot_dim is negative"; return nullptr; }
             if (!latent_attn_shape_ok(L.kv_rank, L.rot)) { err = "latent attention: kv_rank " + std::to_string(L.kv_rank) + " (+ rot_dim) is beyond what the attention kernel holds per lane (1088)"; return nullptr; }
             L.scale = (float)mx["scale"].as_double(1.0);
             const Json &mask = mx["mask"];
@@ -243,14 +191,14 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
             if (kind == "dense") {
                 L.ff_kind = NVX_FF_DENSE;
                 L.ff = (int)mlp["ff"].as_int();
-                if (!positive(err, "mlp.ff", L.ff)) return nullptr;
+                if (!cfg_positive(err, "mlp.ff", L.ff)) return nullptr;
                 L.up = ld.rows({{pf + "up", L.ff}}, W);
                 L.down_ff = ld.rows({{pf + "down", W}}, L.ff);
             } else if (kind == "moe") {
                 L.ff_kind = NVX_FF_EXPERTS;
                 L.ff = (int)mlp["expert"]["ff"].as_int();
                 L.n_expert = (int)mlp["router"]["experts"].as_int(); L.top = (int)mlp["router"]["top"].as_int();
-                if (!positive(err, "mlp.expert.ff", L.ff) || !positive(err, "mlp.router.experts", L.n_expert, 4096) || !positive(err, "mlp.router.top", L.top, L.n_expert)) return nullptr;
+                if (!cfg_positive(err, "mlp.expert.ff", L.ff) || !cfg_positive(err, "mlp.router.experts", L.n_expert, 4096) || !cfg_positive(err, "mlp.router.top", L.top, L.n_expert)) return nullptr;
                 std::vector<std::pair<std::string, int>> g, u, d;
                 for (int e = 0; e < L.n_expert; e++) {
                     const std::string pe = pf + "e" + std::to_string(e) + ".";
@@ -271,22 +219,13 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
     }
     if (!ld.err.empty()) { err = ld.err; return nullptr; }
 
-    // the order of layer runs: layers before the looped span once, the span `times` times (each pass opens with the input projection), the rest once
-    int a = 0, b = 0, times = 0;
-    const Json &loop = cfg["loop"];
-    if (loop.is_object()) {
-        a = (int)loop["start"].as_int(0); b = (int)loop["stop"].as_int(0); times = (int)loop["times"].as_int(1);
-        if (a < 0 || b > nl || times < 0 || times > 4096) { err = "configuration: loop start / stop / times out of range"; return nullptr; }
-        if (b <= a || times < 1) { a = b = 0; times = 0; }
-    }
-    const auto add_run = [&](int il, int pass) {
-        NvxRun r; r.layer = il; r.pass = pass;
-        r.plane = M.layers[(size_t)il].type == NVX_LATENT ? M.n_latent_runs++ : M.n_mlstm_runs++;
-        M.runs.push_back(r);
-    };
-    for (int i = 0; i < a; i++) add_run(i, -1);
-    for (int t = 0; t < times; t++) for (int i = a; i < b; i++) add_run(i, i == a ? t : -1);
-    for (int i = b; i < nl; i++) add_run(i, -1);
+    // the order of layer runs; every pass of the looped span opens with the input projection
+    int times = 0;
+    if (!cfg_layer_runs(cfg["loop"], nl, err, times, [&](int il, int pass) {
+            NvxRun r; r.layer = il; r.pass = pass;
+            r.plane = M.layers[(size_t)il].type == NVX_LATENT ? M.n_cache_runs++ : M.n_mlstm_runs++;
+            M.runs.push_back(r);
+        })) return nullptr;
     if (times > 0) {
         M.loop_in = ld.rows({{"loop.in", W}}, 2 * W);
         if (const SafeTensor *t = ld.need("loop.step", "BF16", {times, W})) {
@@ -297,19 +236,14 @@ Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int 
         }
     }
     if (!ld.err.empty()) { err = ld.err; return nullptr; }
-    if (hipDeviceSynchronize() != hipSuccess) { err = "device synchronise failed after the upload"; status = -103; return nullptr; }
-
     HParams &hp = m->hp;
     hp.arch = "novorax";
     hp.n_embd = W; hp.n_vocab = V; hp.n_vocab_local = V; hp.n_layer = nl; hp.n_layer_runs = (int)M.runs.size();
     hp.n_head = M.layers[0].heads; hp.n_head_kv = 1; hp.head_dim = M.layers[0].dim; hp.eps = M.eps;
     hp.n_head_full = hp.n_head; hp.n_head_kv_full = 1;
-    m->device_bytes = ld.bytes;
-    m->file_tensor_bytes = ld.st.file_bytes();
-    m->bytes_per_token = ld.bytes;
     m->desc = "novorax " + std::to_string(nl) + " layers (" + std::to_string(M.runs.size()) + " runs) width " + std::to_string(W) + " BF16";
     status = 0;
-    return m.release();
+    return m;
 }
 
 // ------------------------------------------------------------------------------------------ context
@@ -329,17 +263,17 @@ bool Context::init_novorax(std::string &err) {
     d_tok_ = (int32_t *)(d_stage_ + 16);
     d_pos_ = d_tok_ + Tp; d_seq_ = d_pos_ + Tp; d_cell_ = d_seq_ + Tp; d_outrow_ = d_cell_ + Tp;
     d_seqmask_ = (uint64_t *)(d_outrow_ + Tp);
-    d_seg_ = (int32_t *)dalloc(4 * T * 4);
-    if (!d_seg_ || hipHostMalloc((void **)&h_seg_, 4 * T * 4, hipHostMallocDefault) != hipSuccess) { err = "segment list allocation failed"; return false; }
+    d_seg_ = (int32_t *)dalloc(5 * T * 4);
+    if (!d_seg_ || hipHostMalloc((void **)&h_seg_, 5 * T * 4, hipHostMallocDefault) != hipSuccess) { err = "segment list allocation failed"; return false; }
 
     // cache planes and recurrent state
-    nvx_cache_.assign((size_t)M.n_latent_runs, nullptr);
+    nvx_cache_.assign((size_t)M.n_cache_runs, nullptr);
     nvx_S_.assign((size_t)M.n_mlstm_runs, nullptr); nvx_n_ = nvx_S_; nvx_m_ = nvx_S_;
     for (const NvxRun &r : M.runs) {
         const NvxLayer &L = M.layers[(size_t)r.layer];
-        if (L.type == NVX_LATENT) {
-            nvx_cache_[(size_t)r.plane] = (float *)dalloc(NC * (size_t)(L.kv_rank + L.rot) * 4);
-            if (!nvx_cache_[(size_t)r.plane]) { err = "latent cache allocation failed"; return false; }
+        if (L.type != NVX_MLSTM) {
+            nvx_cache_[(size_t)r.plane] = (float *)dalloc(NC * (size_t)L.cache_row() * 4);
+            if (!nvx_cache_[(size_t)r.plane]) { err = "attention cache allocation failed"; return false; }
         } else {
             const size_t HS = (size_t)L.heads;
             nvx_S_[(size_t)r.plane] = (float *)dalloc(NS * HS * L.dim * L.vdim * 4);
@@ -366,8 +300,8 @@ bool Context::init_novorax(std::string &err) {
     nvx_o_ = (float *)dalloc(T * (size_t)std::max(M.max_att, 1) * 4);
     nvx_ff_ = (float *)dalloc(T * TOP * (size_t)std::max(M.max_ff, 1) * 4);
     {
-        int kr = 1;
-        for (const NvxLayer &L : M.layers) if (L.type == NVX_LATENT) kr = std::max(kr, L.kv_rank);
+        int kr = 1;                                              // widest record of a split attention scan: the latent, or a value head
+        for (const NvxLayer &L : M.layers) kr = std::max(kr, L.type == NVX_LATENT ? L.kv_rank : L.type == NVX_GQ ? L.vdim : 1);
         nvx_part_ = (float *)dalloc((size_t)LATENT_ATTN_SPLIT_MAX_PAIRS * LATENT_ATTN_SPLITS * (size_t)(kr + 2) * 4);
     }
     if (!x_ || !xn_ || !xo_ || !nvx_x0_ || !nvx_xcat_ || !nvx_y_ || !nvx_a_ || !nvx_cq_ || !nvx_q_ || !nvx_qa_ || !nvx_lat_ || !nvx_att_ || !nvx_o_ || !nvx_ff_) { err = "activation buffer allocation failed"; return false; }
@@ -378,7 +312,13 @@ bool Context::init_novorax(std::string &err) {
         nvx_meta_ = (int32_t *)dalloc((size_t)(2 * M.max_expert + 1) * 4);
         nvx_slot_ = (int32_t *)dalloc(T * TOP * 4);
         nvx_tokof_ = (int32_t *)dalloc(T * TOP * 4);
-        if (!nvx_xg_ || !nvx_yg_ || !nvx_ids_ || !nvx_meta_ || !nvx_slot_ || !nvx_tokof_) { err = "expert batch buffers allocation failed"; return false; }
+        nvx_rw_ = (float *)dalloc(T * TOP * 4);
+        if (!nvx_xg_ || !nvx_yg_ || !nvx_ids_ || !nvx_meta_ || !nvx_slot_ || !nvx_tokof_ || !nvx_rw_) { err = "expert batch buffers allocation failed"; return false; }
+    }
+    if (M.max_shared_ff > 0) {
+        nvx_sh_ = (float *)dalloc(T * (size_t)M.max_shared_ff * 4);
+        nvx_ys_ = (float *)dalloc(T * W * 4);
+        if (!nvx_sh_ || !nvx_ys_) { err = "shared expert buffers allocation failed"; return false; }
     }
     d_argmax_ = (int32_t *)dalloc(T * 4);
     argmax_scratch_ = (float *)dalloc(T * 129 * 4);
@@ -426,9 +366,21 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, 
     {
         // per token: one past the highest cell its attention can need - the sequence's cells from earlier batches, and this batch's own cells up to the token
         // (positions grow along a sequence's rows of a batch; a row that breaks that order falls back to the high-water mark)
-        int32_t *hi = h_seg_ + 3 * T;
-        int base[64], last_pos[64];
-        for (int s = 0; s < 64; s++) { base[s] = 0; last_pos[s] = -1; }
+        // and the lowest cell that can still lie inside the widest window of any of the sequence's tokens in this batch (its earliest token decides; cells
+        // of no use to a later token cost it a visibility test each)
+        int32_t *hi = h_seg_ + 3 * T, *lo = h_seg_ + 4 * T;
+        int base[64], last_pos[64], first_pos[64], low[64];
+        for (int s = 0; s < 64; s++) { base[s] = 0; last_pos[s] = -1; first_pos[s] = 0x7fffffff; low[s] = (int)cells_.size(); }
+        const int win = model->nvx->max_window;
+        if (win > 0) {
+            for (int i = 0; i < n; i++) first_pos[seq[i] & 63] = std::min(first_pos[seq[i] & 63], (int)pos[i]);
+            for (size_t c = 0; c < cells_.size(); c++) {
+                if (cells_[c].pos < 0) continue;
+                uint64_t mk = cells_[c].seqs;
+                while (mk) { const int s = __builtin_ctzll(mk); mk &= mk - 1; if (first_pos[s] != 0x7fffffff && cells_[c].pos > first_pos[s] - win && (int)c < low[s]) low[s] = (int)c; }
+            }
+        }
+        for (int i = 0; i < n; i++) lo[i] = win > 0 ? low[seq[i] & 63] : 0;
         std::vector<char> mine(cells_.size(), 0);
         for (int i = 0; i < n; i++) mine[(size_t)tcell[i]] = 1;
         for (size_t c = 0; c < cells_.size(); c++) {
@@ -461,17 +413,17 @@ bool Context::nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, 
         seen |= bit;
     }
     if (ns > first) nvx_waves_.push_back({first, ns - first});
-    return hipMemcpyAsync(d_seg_, h_seg_, 4 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
+    return hipMemcpyAsync(d_seg_, h_seg_, 5 * T * 4, hipMemcpyHostToDevice, stream_) == hipSuccess;
 }
 
-// pn != nullptr: the rows of x are RMS-normed with weight (1 + pn) on the way in (few rows: inside the launch; batches: a norm launch into xn_ first)
+// pn != nullptr: the rows of x are RMS-normed with weight (norm_off + pn) on the way in (few rows: inside the launch; batches: a norm launch into xn_ first)
 hipError_t Context::nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi, const BfMat *w2, float out_scale, const float *pn) {
     MMBArgs a;
     if (pn && T > MMB_VEC_ROWS) {
-        NVX_TRY(launch_rmsnorm_f32(x, ldx, pn, 1.0f, nullptr, xn_, w.K, w.K, T, model->nvx->eps, stream_));
+        NVX_TRY(launch_rmsnorm_f32(x, ldx, pn, model->nvx->norm_off, nullptr, xn_, w.K, w.K, T, model->nvx->eps, stream_));
         x = xn_; ldx = w.K; pn = nullptr;
     }
-    a.pn_w = pn; a.pn_off = 1.0f; a.pn_eps = model->nvx->eps;
+    a.pn_w = pn; a.pn_off = model->nvx->norm_off; a.pn_eps = model->nvx->eps;
     a.x = x; a.ldx = ldx; a.w = w.w; a.w2 = w2 ? w2->w : nullptr; a.ldw = w.K; a.y = y; a.ldy = ldy;
     a.T = T; a.N = w.N; a.K = w.K; a.epi = epi; a.f32 = cp.exact_f32 ? 1 : 0; a.out_scale = out_scale;
     return launch_mmb(a, stream_);
@@ -536,6 +488,12 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(launch_add_row(x_, M.loop_step + (size_t)r.pass * W, W, T, stream_));
         }
         const int H = L.heads;
+        if (M.parallel_block) {
+            NVX_TRY(nvx_parallel_block(L, r, T));
+            if (debug_taps_ && dbg_) NVX_TRY(hipMemcpyAsync(dbg_ + (size_t)ir * cp.n_ubatch * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, stream_));
+            ir++;
+            continue;
+        }
         if (L.type == NVX_LATENT) {
             const int QD = L.dim + L.rot, KR = L.kv_rank, LD_A = L.q_rank + KR + L.rot;
             float *cache = nvx_cache_[(size_t)r.plane];
@@ -564,7 +522,7 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(launch_mmb(ua, stream_));
             NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
             prof_mark("latent_attention");
-        } else {
+        } else if (L.type == NVX_MLSTM) {
             const int LD_P = L.proj.N;
             NVX_TRY(nvx_linear(L.proj, x_, W, T, nvx_a_, LD_P, MMB_STORE, nullptr, 1.0f, L.norm1));
             MlstmArgs ma{};
@@ -579,7 +537,7 @@ hipError_t Context::run_layers_novorax(int T) {
             NVX_TRY(launch_mlstm_out(nvx_o_, H * L.vdim, nvx_a_, LD_P, 2 * H * L.dim + H * L.vdim, L.mix_norm, T, H, L.vdim, eps, nvx_att_, H * L.vdim, stream_));
             NVX_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
             prof_mark("mlstm");
-        }
+        } else return hipErrorInvalidValue;                      // (a mixer this block form has no path for: refused at load)
         NVX_TRY(launch_rmsnorm_f32(nvx_y_, W, L.norm1b, 1.0f, x_, x_, W, W, T, eps, stream_));
         if (L.ff_kind != NVX_FF_NONE) {
             NVX_TRY(nvx_feed_forward(L, T));

@@ -58,10 +58,10 @@ static bool type_supported(int t) {
 Model *model_load(const std::string &path, int main_gpu, std::string &err, int &status, int prefill_planes, int tp_rank, int tp_size) {
     status = 0;
     {
-        std::string dir;                                        // a folder with config.json + model.safetensors: the Novorax loader (novorax.cc)
-        if (novorax_path(path, dir)) {
-            if (tp_size > 1) { err = "row split of a Novorax model is not supported"; status = -102; return nullptr; }
-            return novorax_load(dir, main_gpu, err, status);
+        std::string dir;                                        // a folder with config.json + model.safetensors: the loader its architecture names (novorax.cc)
+        if (config_model_path(path, dir)) {
+            if (tp_size > 1) { err = "row split of a folder model (config.json + safetensors) is not supported"; status = -102; return nullptr; }
+            return config_model_load(dir, main_gpu, err, status);
         }
     }
     std::unique_ptr<Model> m(new Model());
@@ -1942,7 +1942,7 @@ int Context::decode_ubatch(int n, const int32_t *tokens, const int32_t *pos, con
 
     const int V = model->hp.n_vocab;
     const bool nvx = model->nvx != nullptr;
-    if (nvx && ub_embd_) { last_error = "a Novorax model takes token ids, not embeddings"; return -1; }
+    if (nvx && ub_embd_) { last_error = "a folder model (config.json + safetensors) takes token ids, not embeddings"; return -1; }
     const auto layers_of = [&](int T, int cap) { return nvx ? run_layers_novorax(T) : run_layers(T, cap); };
     const auto output_of = [&](int rows, int base) { return nvx ? run_output_novorax(rows, base) : run_output(rows, base); };
     if (n == 1 && !model->hp.encoder && !ub_embd_ && !nvx) { (void)mega_prepare(); (void)engine_prepare(); }   // allocate and upload on first use: must not happen inside a stream capture

@@ -74,7 +74,7 @@ struct Model {
     DevTensor tok_embd, out_norm, output, rope_freqs;
     DevTensor tok_types, tok_norm, tok_norm_b;       // encoder files: token-type table (row 0 is added to every token), LayerNorm of the embeddings
     std::vector<LayerWeights> layers;
-    std::unique_ptr<NovoraxModel> nvx;  // architecture "Novorax" (a folder with config.json + model.safetensors): its own layer stack, see novorax.h
+    std::unique_ptr<NovoraxModel> nvx;  // a folder model (config.json + model.safetensors; architectures Novorax, Fidepel): its own layer stack, see novorax.h
     uint64_t device_bytes = 0, host_bytes = 0, file_tensor_bytes = 0, bytes_per_token = 0, planes_bytes = 0;
     ~Model();
 };
@@ -82,9 +82,10 @@ struct Model {
 // prefill_planes: 0 = never, 1 = always (fails when memory is short), -1 = when device memory allows (default)
 // tp_size > 1: load rank tp_rank's slice of every projection (rows of attn_q/k/v, ffn_gate/up and output; the matching
 // super-block columns of attn_output and ffn_down), cut on head and 256-element boundaries
-// a folder (or its config.json) whose "architecture" is Novorax: weights to the device, layer runs laid out (novorax.cc)
-Model *novorax_load(const std::string &dir, int main_gpu, std::string &err, int &status);
-bool novorax_path(const std::string &path, std::string &dir);   // does `path` name such a folder
+// a folder (or its config.json) with model.safetensors beside it: the loader of the design its "architecture" names puts the weights on the device and lays
+// out the layer runs (novorax.cc config_model_load: Novorax, Fidepel)
+Model *config_model_load(const std::string &dir, int main_gpu, std::string &err, int &status);
+bool config_model_path(const std::string &path, std::string &dir);   // does `path` name such a folder
 Model *model_load(const std::string &path, int main_gpu, std::string &err, int &status, int prefill_planes = -1, int tp_rank = 0, int tp_size = 1);
 
 struct KVCell {
@@ -183,18 +184,23 @@ class Context {
     hipError_t nvx_linear(const BfMat &w, const float *x, int ldx, int T, float *y, int ldy, int epi = MMB_STORE, const BfMat *w2 = nullptr, float out_scale = 1.0f,
                           const float *pn = nullptr);
     hipError_t nvx_feed_forward(const NvxLayer &L, int T);
+    // fidepel.cc: a block whose mixer and feed-forward read one norm; grouped-query attention on the run's cache plane; experts picked by a router
+    hipError_t nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T);
+    hipError_t nvx_gq_attention(const NvxLayer &L, const NvxRun &r, const float *h, const float *pn, int T);
+    hipError_t nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T);
+    float *nvx_sh_ = nullptr, *nvx_ys_ = nullptr, *nvx_rw_ = nullptr;   // shared expert's hidden rows and output; router weights [T][top]
     // runs of consecutive tokens of one sequence -> segment arrays; per-token scan bounds of the attention (pinned, then device)
     bool nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, const int *tcell);
     void nvx_state_reset(int seq);                          // seq < 0: every slot
     void nvx_state_copy(int src, int dst);
-    std::vector<float *> nvx_cache_;                        // [latent run] [n_ctx][kv_rank + rot]
+    std::vector<float *> nvx_cache_;                        // [attention run] [n_ctx][the layer's cache_row()]
     std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [mlstm run] [n_seq_max][H][D][VD], [..][H][D], [..][H]
     std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
     float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
     float *nvx_part_ = nullptr;                             // split records of the latent attention of single-token steps
     float *nvx_att_ = nullptr, *nvx_o_ = nullptr, *nvx_ff_ = nullptr, *nvx_xg_ = nullptr, *nvx_yg_ = nullptr;
     int32_t *nvx_ids_ = nullptr, *nvx_meta_ = nullptr, *nvx_slot_ = nullptr, *nvx_tokof_ = nullptr;
-    int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [4][n_ubatch]: start, length, slot of every segment; scan bound of every token
+    int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [5][n_ubatch]: start, length, slot of every segment; upper and lower scan bound of every token
     std::vector<std::pair<int, int>> nvx_waves_;            // segment ranges [first, count) that may share a launch (no slot twice)
     hipError_t run_output(int n_out, int out_base);
     hipError_t linear(const DevTensor &w, const ActQuant &aq, const float *x_f32, int K, int T, float *out, int ld_out,
