@@ -28,8 +28,11 @@ __device__ float gq_block_sum_256(float v, float *sh) {
     return (sh[0] + sh[1]) + (sh[2] + sh[3]);
 }
 
+constexpr int GQ_MAX_D = 256;                                   // dim and vdim the attention kernel is instantiated for (4 x 64)
+
 __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     __shared__ float sh[4];
+    __shared__ float cs[2][GQ_MAX_D / 2];                       // cos / sin of the token's angle per pair: computed once, read by every head
     const int t = blockIdx.x, tid = threadIdx.x;
     const int NQ = a.H * a.dim, NK = a.G * a.dim, NV = a.G * a.vdim, half = a.rot_dims >> 1;
     const float *qr = a.p + (size_t)t * a.ld_p, *kr = qr + NQ, *vr = kr + NK;
@@ -45,6 +48,8 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         inv_k = 1.0f / sqrtf(gq_block_sum_256(ss, sh) / (float)NK + a.eps);
     }
     const float p = (float)a.tok_pos[t];
+    if (tid < half) { const float ang = p * a.rot_freq[tid]; cs[0][tid] = cosf(ang); cs[1][tid] = sinf(ang); }
+    __syncthreads();
     float *qo = a.q + (size_t)t * a.ld_q;
     float *row = a.cache + (size_t)a.tok_cell[t] * (size_t)(NK + NV);
     // one loop over the query entries, then the key entries: element (head, d) of either
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
         float o;
         if (d < a.rot_dims) {
             const int j = d < half ? d : d - half;
-            const float ang = p * a.rot_freq[j], c = cosf(ang), s = sinf(ang);
+            const float c = cs[0][j], s = cs[1][j];
             float u = src[b + j] * inv, w = src[b + j + half] * inv;
             if (wn) { u *= wn[b + j]; w *= wn[b + j + half]; }
             o = d < half ? u * c - w * s : w * c + u * s;
@@ -73,8 +78,6 @@ __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     }
     for (int i = tid; i < NV; i += 256) row[NK + i] = vr[i];
 }
-
-constexpr int GQ_MAX_D = 256;                                   // dim and vdim the attention kernel is instantiated for (4 x 64)
 
 // One workgroup per (token, head), NW waves.  A wave works on four cells at a time: each 16-lane group owns one cell, its lanes hold elements
 // 64 j + 4 li .. + 3 of the key head and of the value head (16-byte loads) and the matching running sums; the next four cells of the wave are requested
@@ -242,13 +245,200 @@ static hipError_t launch_gq_attn_nj(const GqAttnArgs &a, hipStream_t st) {
     return hipGetLastError();
 }
 
+
+// ---- prompt batches: the same attention as one LDS-tiled pass per (tile of 64 batch rows, head)
+// The tile's rows may belong to any sequences at any positions: visibility is decided per (row, cell) pair from the cell table, exactly as above.  The
+// scanned cells are walked in blocks of 64; a block none of whose cells can be seen by any row of the tile (wrong sequence, beyond the tile's last position,
+// before its first window) costs one read of its cell table entries.  Per block: S = Q K^T in 32-wide slices of the head (both operands through LDS, a
+// thread owns 4 rows x 4 cells), the running softmax per row (16 lanes share a row), P to LDS, O += P V in 64-column slices of the value head (a thread
+// owns 4 rows x 4 columns per slice).  NVC = ceil(vdim / 64).  dim and vdim multiples of 4.
+constexpr int GQT_B = 64, GQT_DC = 32, GQT_LDQ = GQT_DC + 4, GQT_LDP = GQT_B + 4;
+constexpr size_t GQT_LDS_FLOATS = 2 * GQT_B * GQT_LDQ + 2 * GQT_B * GQT_LDP + 5 * GQT_B;
+
+template <int NVC>
+__global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
+    extern __shared__ float lds[];
+    float *Qc = lds, *Kc = Qc + GQT_B * GQT_LDQ, *P = Kc + GQT_B * GQT_LDQ, *Vc = P + GQT_B * GQT_LDP;
+    int *rpos = reinterpret_cast<int *>(Vc + GQT_B * GQT_LDP), *rseq = rpos + GQT_B, *cpos = rseq + GQT_B;
+    uint64_t *cseq = reinterpret_cast<uint64_t *>(cpos + GQT_B);
+    __shared__ int red[4];
+    const int D = a.dim, VD = a.vdim, tid = threadIdx.x, tq = tid >> 4, tc = tid & 15;
+    const int row0 = blockIdx.x * GQT_B, h = blockIdx.y, kvh = h / (a.H / a.G);
+    const size_t L = (size_t)a.G * (D + VD), koff = (size_t)kvh * D, voff = (size_t)a.G * D + (size_t)kvh * VD;
+    const int n_kv = *a.n_kv_dev;
+    // the tile's rows: position and sequence of each; over the tile: first and last position, the union of sequences, the range of cells to walk
+    int my_lo = 0x7fffffff, my_hi = 0, my_pmin = 0x7fffffff, my_pmax = -1;
+    if (tid < GQT_B) {
+        const int r = row0 + tid;
+        const bool live = r < a.T;
+        rpos[tid] = live ? a.tok_pos[r] : -1;
+        rseq[tid] = live ? (a.tok_seq[r] & 63) : -1;
+        if (live) {
+            my_pmin = my_pmax = rpos[tid];
+            my_lo = a.tok_lo ? a.tok_lo[r] : 0;
+            my_hi = a.tok_hi ? (a.tok_hi[r] < n_kv ? a.tok_hi[r] : n_kv) : n_kv;
+        }
+    }
+    if (tid < 64) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            my_lo = min(my_lo, __shfl_xor(my_lo, o, 64)); my_hi = max(my_hi, __shfl_xor(my_hi, o, 64));
+            my_pmin = min(my_pmin, __shfl_xor(my_pmin, o, 64)); my_pmax = max(my_pmax, __shfl_xor(my_pmax, o, 64));
+        }
+        if (tid == 0) { red[0] = my_lo; red[1] = my_hi; red[2] = my_pmin; red[3] = my_pmax; }
+    }
+    __syncthreads();
+    const int c_begin = red[0] < red[1] ? red[0] : red[1], c_end = red[1], pmin = red[2], pmax = red[3];
+    uint64_t seqs = 0;
+    for (int r = 0; r < GQT_B; r++) if (rseq[r] >= 0) seqs |= 1ull << rseq[r];
+    float s[4][4], o[4][NVC * 4], m[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        m[i] = -INFINITY; l[i] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < NVC * 4; e++) o[i][e] = 0.0f;
+    }
+    for (int c0 = c_begin; c0 < c_end; c0 += GQT_B) {
+        __syncthreads();                                        // (the previous block's P / V / cell entries are no longer read)
+        int any = 0;
+        if (tid < GQT_B) {
+            const int c = c0 + tid;
+            int cp = -1; uint64_t cs = 0;
+            if (c < c_end) { cp = a.cell_pos[c]; cs = a.cell_seq[c]; }
+            cpos[tid] = cp; cseq[tid] = cs;
+            any = cp >= 0 && cp <= pmax && (cs & seqs) != 0 && !(a.window > 0 && pmin - cp >= a.window);
+        }
+        if (!__syncthreads_or(any)) continue;
+        // ---- S = Q K^T
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) s[i][j] = 0.0f;
+        for (int dc = 0; dc < D; dc += GQT_DC) {
+            if (dc > 0) __syncthreads();
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int idx = tid + 256 * k, r = idx >> 3, d = dc + (idx & 7) * 4;
+                float4 qv = make_float4(0.0f, 0.0f, 0.0f, 0.0f), kv = qv;
+                if (d < D) {
+                    if (row0 + r < a.T) qv = *reinterpret_cast<const float4 *>(a.q + (size_t)(row0 + r) * a.ld_q + (size_t)h * D + d);
+                    if (cpos[r] >= 0) kv = *reinterpret_cast<const float4 *>(a.cache + (size_t)(c0 + r) * L + koff + d);
+                }
+                *reinterpret_cast<float4 *>(Qc + r * GQT_LDQ + (idx & 7) * 4) = qv;
+                *reinterpret_cast<float4 *>(Kc + r * GQT_LDQ + (idx & 7) * 4) = kv;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int d4 = 0; d4 < GQT_DC / 4; d4++) {
+                float4 qf[4], kf[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) qf[i] = *reinterpret_cast<const float4 *>(Qc + (tq * 4 + i) * GQT_LDQ + d4 * 4);
+#pragma unroll
+                for (int j = 0; j < 4; j++) kf[j] = *reinterpret_cast<const float4 *>(Kc + (tc + 16 * j) * GQT_LDQ + d4 * 4);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        s[i][j] = fmaf(qf[i].x, kf[j].x, s[i][j]); s[i][j] = fmaf(qf[i].y, kf[j].y, s[i][j]);
+                        s[i][j] = fmaf(qf[i].z, kf[j].z, s[i][j]); s[i][j] = fmaf(qf[i].w, kf[j].w, s[i][j]);
+                    }
+            }
+        }
+        // ---- the running softmax of each row; P to LDS
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = tq * 4 + i, rp = rpos[r];
+            const uint64_t rbit = rseq[r] >= 0 ? 1ull << rseq[r] : 0ull;
+            bool vis[4];
+            float bm = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int cp = cpos[tc + 16 * j];
+                vis[j] = cp >= 0 && cp <= rp && (cseq[tc + 16 * j] & rbit) != 0 && !(a.window > 0 && rp - cp >= a.window);
+                if (vis[j]) bm = fmaxf(bm, s[i][j]);
+            }
+#pragma unroll
+            for (int of = 8; of > 0; of >>= 1) bm = fmaxf(bm, __shfl_xor(bm, of, 64));
+            const float mn = fmaxf(m[i], bm);
+            const float alpha = m[i] == -INFINITY ? 0.0f : expf(m[i] - mn);   // (mn = -inf only while m is: nothing seen yet, nothing to scale)
+            float ps = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float pj = vis[j] ? expf(s[i][j] - mn) : 0.0f;
+                ps += pj;
+                P[r * GQT_LDP + tc + 16 * j] = pj;
+            }
+#pragma unroll
+            for (int of = 8; of > 0; of >>= 1) ps += __shfl_xor(ps, of, 64);
+            l[i] = l[i] * alpha + ps;
+            m[i] = mn;
+#pragma unroll
+            for (int e = 0; e < NVC * 4; e++) o[i][e] *= alpha;
+        }
+        // ---- O += P V
+#pragma unroll
+        for (int vc = 0; vc < NVC; vc++) {
+            __syncthreads();                                    // (P is complete; the previous slice of V has been used)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int idx = tid + 256 * k, r = idx >> 4, col = vc * 64 + (idx & 15) * 4;
+                float4 vv = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (col < VD && cpos[r] >= 0) vv = *reinterpret_cast<const float4 *>(a.cache + (size_t)(c0 + r) * L + voff + col);
+                *reinterpret_cast<float4 *>(Vc + r * GQT_LDP + (idx & 15) * 4) = vv;
+            }
+            __syncthreads();
+            for (int c = 0; c < GQT_B; c += 4) {
+                float4 pf[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) pf[i] = *reinterpret_cast<const float4 *>(P + (tq * 4 + i) * GQT_LDP + c);
+#pragma unroll
+                for (int cc = 0; cc < 4; cc++) {
+                    const float4 vf = *reinterpret_cast<const float4 *>(Vc + (c + cc) * GQT_LDP + tc * 4);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float pw = cc == 0 ? pf[i].x : cc == 1 ? pf[i].y : cc == 2 ? pf[i].z : pf[i].w;
+                        o[i][vc * 4 + 0] = fmaf(pw, vf.x, o[i][vc * 4 + 0]); o[i][vc * 4 + 1] = fmaf(pw, vf.y, o[i][vc * 4 + 1]);
+                        o[i][vc * 4 + 2] = fmaf(pw, vf.z, o[i][vc * 4 + 2]); o[i][vc * 4 + 3] = fmaf(pw, vf.w, o[i][vc * 4 + 3]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = row0 + tq * 4 + i;
+        if (r >= a.T) continue;
+        float MM = m[i], den = l[i], sc = 1.0f;
+        if (a.sink) {
+            MM = fmaxf(m[i], a.sink[h]);
+            sc = l[i] > 0.0f ? expf(m[i] - MM) : 0.0f;
+            den = l[i] * sc + expf(a.sink[h] - MM);
+        }
+        float inv = den > 0.0f ? sc / den : 0.0f;
+        if (a.gate) inv *= 1.0f / (1.0f + expf(-a.gate[(size_t)r * a.ld_gate + h]));
+#pragma unroll
+        for (int vc = 0; vc < NVC; vc++) {
+            const int col = vc * 64 + tc * 4;
+            if (col < VD) *reinterpret_cast<float4 *>(a.out + (size_t)r * a.ld_out + (size_t)h * VD + col) =
+                make_float4(o[i][vc * 4 + 0] * inv, o[i][vc * 4 + 1] * inv, o[i][vc * 4 + 2] * inv, o[i][vc * 4 + 3] * inv);
+        }
+    }
+}
+
+template <int NVC>
+static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
+    const dim3 grid((unsigned)((a.T + GQT_B - 1) / GQT_B), (unsigned)a.H);
+    hipLaunchKernelGGL((gq_attn_tile_kernel<NVC>), grid, dim3(256), GQT_LDS_FLOATS * sizeof(float), st, a);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 bool gq_attn_shape_ok(int H, int G, int dim, int vdim) { return H >= 1 && G >= 1 && H % G == 0 && dim >= 1 && vdim >= 1 && dim <= GQ_MAX_D && vdim <= GQ_MAX_D; }
 
 hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
-    if (a.rot_dims < 0 || a.rot_dims > a.dim || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
+    if (a.rot_dims < 0 || a.rot_dims > a.dim || a.rot_dims > GQ_MAX_D || (a.rot_dims & 1) || (a.rot_dims > 0 && !a.rot_freq)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(gq_prep_kernel, dim3((unsigned)a.T), dim3(256), 0, st, a);
     return hipGetLastError();
 }
@@ -256,6 +446,13 @@ hipError_t launch_gq_prep(const GqPrepArgs &a, hipStream_t st) {
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
     if (a.T <= 0) return hipSuccess;
     if (!gq_attn_shape_ok(a.H, a.G, a.dim, a.vdim)) return hipErrorInvalidValue;
+    // batches: the tiled pass (16-byte loads everywhere: head sizes, strides and bases must allow them); a few rows: one workgroup per (row, head)
+    const auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (a.T >= GQ_TILE_MIN_ROWS && (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (a.ld_q & 3) == 0 && (a.ld_out & 3) == 0 && al16(a.q) && al16(a.out) && al16(a.cache)) {
+        if (a.vdim <= 64) return launch_gq_attn_tile<1>(a, st);
+        if (a.vdim <= 128) return launch_gq_attn_tile<2>(a, st);
+        return launch_gq_attn_tile<4>(a, st);
+    }
     const int Dm = a.dim > a.vdim ? a.dim : a.vdim;
     if (Dm <= 64) return launch_gq_attn_nj<1>(a, st);
     if (Dm <= 128) return launch_gq_attn_nj<2>(a, st);

@@ -321,6 +321,7 @@ struct GqAttnArgs {
     // lowest cell that can hold one still inside the window
     const int32_t *tok_hi, *tok_lo;
 };
+constexpr int GQ_TILE_MIN_ROWS = 32;     // batches from this many rows on take the LDS-tiled pass (64 rows x 64 cells per step) instead of one workgroup per (row, head)
 bool gq_attn_shape_ok(int H, int G, int dim, int vdim);
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st);
 
