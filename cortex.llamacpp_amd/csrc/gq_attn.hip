@@ -28,7 +28,7 @@ __device__ float gq_block_sum_256(float v, float *sh) {
     return (sh[0] + sh[1]) + (sh[2] + sh[3]);
 }
 
-constexpr int GQ_MAX_D = 256;                                   // dim and vdim the attention kernel is instantiated for (4 x 64)
+constexpr int GQ_MAX_D = 512;                                   // dim and vdim the attention kernel is instantiated for (8 x 64)
 
 __global__ __launch_bounds__(256) void gq_prep_kernel(GqPrepArgs a) {
     __shared__ float sh[4];
@@ -237,7 +237,7 @@ static hipError_t launch_gq_attn_nj(const GqAttnArgs &a, hipStream_t st) {
     const int nw = (long long)a.T * a.H <= 1024 ? 8 : 4;
     const size_t lds = (size_t)(NJ * 64 + 2 * nw + nw * NJ * 64) * sizeof(float);
     const bool vec = (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (reinterpret_cast<uintptr_t>(a.cache) & 15) == 0;
-    const int splits = a.part && a.splits > 1 ? a.splits : 1;
+    const int splits = a.part && a.splits > 1 && (size_t)a.T * a.H * a.splits * (a.vdim + 2) <= a.part_floats ? a.splits : 1;
     const dim3 grid((unsigned)a.T, (unsigned)a.H, (unsigned)splits);
     if (vec) hipLaunchKernelGGL((gq_attn_kernel<NJ, true>), grid, dim3(64 * nw), lds, st, a);
     else hipLaunchKernelGGL((gq_attn_kernel<NJ, false>), grid, dim3(64 * nw), lds, st, a);
@@ -246,29 +246,31 @@ static hipError_t launch_gq_attn_nj(const GqAttnArgs &a, hipStream_t st) {
 }
 
 
-// ---- prompt batches: the same attention as one LDS-tiled pass per (tile of 64 batch rows, head)
+// ---- prompt batches: the same attention as one LDS-tiled pass per (tile of 16 * RPT batch rows, head)
 // The tile's rows may belong to any sequences at any positions: visibility is decided per (row, cell) pair from the cell table, exactly as above.  The
 // scanned cells are walked in blocks of 64; a block none of whose cells can be seen by any row of the tile (wrong sequence, beyond the tile's last position,
 // before its first window) costs one read of its cell table entries.  Per block: S = Q K^T in 32-wide slices of the head (both operands through LDS, a
-// thread owns 4 rows x 4 cells), the running softmax per row (16 lanes share a row), P to LDS, O += P V in 64-column slices of the value head (a thread
-// owns 4 rows x 4 columns per slice).  NVC = ceil(vdim / 64).  dim and vdim multiples of 4.
+// thread owns RPT rows x 4 cells), the running softmax per row (16 lanes share a row), P to LDS, O += P V in 64-column slices of the value head (a thread
+// owns RPT rows x 4 columns per slice).  NVC = ceil(vdim / 64).  dim and vdim multiples of 4.  RPT = 4 (64-row tiles) where that still gives the device
+// two workgroups per CU, else 2: a short prompt is bound by the chain of blocks one workgroup walks, not by arithmetic.
 constexpr int GQT_B = 64, GQT_DC = 32, GQT_LDQ = GQT_DC + 4, GQT_LDP = GQT_B + 4;
-constexpr size_t GQT_LDS_FLOATS = 2 * GQT_B * GQT_LDQ + 2 * GQT_B * GQT_LDP + 5 * GQT_B;
+constexpr size_t gqt_lds_floats(int rows) { return (size_t)(rows + GQT_B) * GQT_LDQ + (size_t)(rows + GQT_B) * GQT_LDP + 2 * rows + 3 * GQT_B; }
 
-template <int NVC>
+template <int NVC, int RPT>
 __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
+    constexpr int BQ = 16 * RPT;
     extern __shared__ float lds[];
-    float *Qc = lds, *Kc = Qc + GQT_B * GQT_LDQ, *P = Kc + GQT_B * GQT_LDQ, *Vc = P + GQT_B * GQT_LDP;
-    int *rpos = reinterpret_cast<int *>(Vc + GQT_B * GQT_LDP), *rseq = rpos + GQT_B, *cpos = rseq + GQT_B;
-    uint64_t *cseq = reinterpret_cast<uint64_t *>(cpos + GQT_B);
+    float *Qc = lds, *Kc = Qc + BQ * GQT_LDQ, *P = Kc + GQT_B * GQT_LDQ, *Vc = P + BQ * GQT_LDP;
+    uint64_t *cseq = reinterpret_cast<uint64_t *>(Vc + GQT_B * GQT_LDP);                     // (an even number of floats in: 8-byte aligned)
+    int *cpos = reinterpret_cast<int *>(cseq + GQT_B), *rpos = cpos + GQT_B, *rseq = rpos + BQ;
     __shared__ int red[4];
     const int D = a.dim, VD = a.vdim, tid = threadIdx.x, tq = tid >> 4, tc = tid & 15;
-    const int row0 = blockIdx.x * GQT_B, h = blockIdx.y, kvh = h / (a.H / a.G);
+    const int row0 = blockIdx.x * BQ, h = blockIdx.y, kvh = h / (a.H / a.G);
     const size_t L = (size_t)a.G * (D + VD), koff = (size_t)kvh * D, voff = (size_t)a.G * D + (size_t)kvh * VD;
     const int n_kv = *a.n_kv_dev;
     // the tile's rows: position and sequence of each; over the tile: first and last position, the union of sequences, the range of cells to walk
     int my_lo = 0x7fffffff, my_hi = 0, my_pmin = 0x7fffffff, my_pmax = -1;
-    if (tid < GQT_B) {
+    if (tid < BQ) {
         const int r = row0 + tid;
         const bool live = r < a.T;
         rpos[tid] = live ? a.tok_pos[r] : -1;
@@ -288,12 +290,18 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
         if (tid == 0) { red[0] = my_lo; red[1] = my_hi; red[2] = my_pmin; red[3] = my_pmax; }
     }
     __syncthreads();
-    const int c_begin = red[0] < red[1] ? red[0] : red[1], c_end = red[1], pmin = red[2], pmax = red[3];
+    int c_begin = red[0] < red[1] ? red[0] : red[1], c_end = red[1];
+    const int pmin = red[2], pmax = red[3];
+    if (gridDim.z > 1) {                                        // the tile's blocks cut into gridDim.z runs, one workgroup each; gq_attn_merge_kernel joins their records
+        const int per = ((c_end - c_begin + GQT_B - 1) / GQT_B + (int)gridDim.z - 1) / (int)gridDim.z * GQT_B;
+        c_begin += (int)blockIdx.z * per;
+        c_end = c_begin + per < c_end ? c_begin + per : c_end;
+    }
     uint64_t seqs = 0;
-    for (int r = 0; r < GQT_B; r++) if (rseq[r] >= 0) seqs |= 1ull << rseq[r];
-    float s[4][4], o[4][NVC * 4], m[4], l[4];
+    for (int r = 0; r < BQ; r++) if (rseq[r] >= 0) seqs |= 1ull << rseq[r];
+    float s[RPT][4], o[RPT][NVC * 4], m[RPT], l[RPT];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < RPT; i++) {
         m[i] = -INFINITY; l[i] = 0.0f;
 #pragma unroll
         for (int e = 0; e < NVC * 4; e++) o[i][e] = 0.0f;
@@ -311,7 +319,7 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
         if (!__syncthreads_or(any)) continue;
         // ---- S = Q K^T
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < RPT; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) s[i][j] = 0.0f;
         for (int dc = 0; dc < D; dc += GQT_DC) {
@@ -321,22 +329,22 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
                 const int idx = tid + 256 * k, r = idx >> 3, d = dc + (idx & 7) * 4;
                 float4 qv = make_float4(0.0f, 0.0f, 0.0f, 0.0f), kv = qv;
                 if (d < D) {
-                    if (row0 + r < a.T) qv = *reinterpret_cast<const float4 *>(a.q + (size_t)(row0 + r) * a.ld_q + (size_t)h * D + d);
+                    if (r < BQ && row0 + r < a.T) qv = *reinterpret_cast<const float4 *>(a.q + (size_t)(row0 + r) * a.ld_q + (size_t)h * D + d);
                     if (cpos[r] >= 0) kv = *reinterpret_cast<const float4 *>(a.cache + (size_t)(c0 + r) * L + koff + d);
                 }
-                *reinterpret_cast<float4 *>(Qc + r * GQT_LDQ + (idx & 7) * 4) = qv;
+                if (r < BQ) *reinterpret_cast<float4 *>(Qc + r * GQT_LDQ + (idx & 7) * 4) = qv;
                 *reinterpret_cast<float4 *>(Kc + r * GQT_LDQ + (idx & 7) * 4) = kv;
             }
             __syncthreads();
 #pragma unroll
             for (int d4 = 0; d4 < GQT_DC / 4; d4++) {
-                float4 qf[4], kf[4];
+                float4 qf[RPT], kf[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) qf[i] = *reinterpret_cast<const float4 *>(Qc + (tq * 4 + i) * GQT_LDQ + d4 * 4);
+                for (int i = 0; i < RPT; i++) qf[i] = *reinterpret_cast<const float4 *>(Qc + (tq * RPT + i) * GQT_LDQ + d4 * 4);
 #pragma unroll
                 for (int j = 0; j < 4; j++) kf[j] = *reinterpret_cast<const float4 *>(Kc + (tc + 16 * j) * GQT_LDQ + d4 * 4);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < RPT; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         s[i][j] = fmaf(qf[i].x, kf[j].x, s[i][j]); s[i][j] = fmaf(qf[i].y, kf[j].y, s[i][j]);
@@ -346,8 +354,8 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
         }
         // ---- the running softmax of each row; P to LDS
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int r = tq * 4 + i, rp = rpos[r];
+        for (int i = 0; i < RPT; i++) {
+            const int r = tq * RPT + i, rp = rpos[r];
             const uint64_t rbit = rseq[r] >= 0 ? 1ull << rseq[r] : 0ull;
             bool vis[4];
             float bm = -INFINITY;
@@ -388,14 +396,14 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
             }
             __syncthreads();
             for (int c = 0; c < GQT_B; c += 4) {
-                float4 pf[4];
+                float4 pf[RPT];
 #pragma unroll
-                for (int i = 0; i < 4; i++) pf[i] = *reinterpret_cast<const float4 *>(P + (tq * 4 + i) * GQT_LDP + c);
+                for (int i = 0; i < RPT; i++) pf[i] = *reinterpret_cast<const float4 *>(P + (tq * RPT + i) * GQT_LDP + c);
 #pragma unroll
                 for (int cc = 0; cc < 4; cc++) {
                     const float4 vf = *reinterpret_cast<const float4 *>(Vc + (c + cc) * GQT_LDP + tc * 4);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
+                    for (int i = 0; i < RPT; i++) {
                         const float pw = cc == 0 ? pf[i].x : cc == 1 ? pf[i].y : cc == 2 ? pf[i].z : pf[i].w;
                         o[i][vc * 4 + 0] = fmaf(pw, vf.x, o[i][vc * 4 + 0]); o[i][vc * 4 + 1] = fmaf(pw, vf.y, o[i][vc * 4 + 1]);
                         o[i][vc * 4 + 2] = fmaf(pw, vf.z, o[i][vc * 4 + 2]); o[i][vc * 4 + 3] = fmaf(pw, vf.w, o[i][vc * 4 + 3]);
@@ -404,9 +412,23 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
             }
         }
     }
+    if (gridDim.z > 1) {                                        // this run's records: maximum, sum, weighted value (sink and gate enter at the merge)
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int r = row0 + tq * 4 + i;
+        for (int i = 0; i < RPT; i++) {
+            const int r = row0 + tq * RPT + i;
+            if (r >= a.T) continue;
+            float *rec = a.part + (((size_t)r * a.H + h) * gridDim.z + blockIdx.z) * (size_t)(VD + 2);
+            if (tc == 0) { rec[0] = m[i]; rec[1] = l[i]; }
+#pragma unroll
+            for (int vc = 0; vc < NVC; vc++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (vc * 64 + tc * 4 + e < VD) rec[2 + vc * 64 + tc * 4 + e] = o[i][vc * 4 + e];
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < RPT; i++) {
+        const int r = row0 + tq * RPT + i;
         if (r >= a.T) continue;
         float MM = m[i], den = l[i], sc = 1.0f;
         if (a.sink) {
@@ -427,8 +449,23 @@ __global__ __launch_bounds__(256) void gq_attn_tile_kernel(GqAttnArgs a) {
 
 template <int NVC>
 static hipError_t launch_gq_attn_tile(const GqAttnArgs &a, hipStream_t st) {
-    const dim3 grid((unsigned)((a.T + GQT_B - 1) / GQT_B), (unsigned)a.H);
-    hipLaunchKernelGGL((gq_attn_tile_kernel<NVC>), grid, dim3(256), GQT_LDS_FLOATS * sizeof(float), st, a);
+    if ((long long)((a.T + 63) / 64) * a.H >= 512) {
+        const dim3 grid((unsigned)((a.T + 63) / 64), (unsigned)a.H);
+        hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 4>), grid, dim3(256), gqt_lds_floats(64) * sizeof(float), st, a);
+        return hipGetLastError();
+    }
+    // too few tiles to fill the device: every tile's chain of cell blocks is cut into runs (at least two blocks each where the cells in use allow), as many
+    // as bring the grid to about four workgroups per CU and as the record buffer holds
+    const long long tiles = (long long)((a.T + 31) / 32) * a.H;
+    long long splits = (1024 + tiles - 1) / tiles;
+    const long long by_blocks = a.n_kv_hint > 0 ? ((a.n_kv_hint + GQT_B - 1) / GQT_B + 1) / 2 : 1;
+    if (splits > by_blocks) splits = by_blocks;
+    if (splits > GQ_TILE_MAX_SPLITS) splits = GQ_TILE_MAX_SPLITS;
+    while (splits > 1 && (!a.part || (size_t)a.T * a.H * splits * (a.vdim + 2) > a.part_floats)) splits--;
+    if (splits < 1) splits = 1;
+    const dim3 grid((unsigned)((a.T + 31) / 32), (unsigned)a.H, (unsigned)splits);
+    hipLaunchKernelGGL((gq_attn_tile_kernel<NVC, 2>), grid, dim3(256), gqt_lds_floats(32) * sizeof(float), st, a);
+    if (splits > 1) hipLaunchKernelGGL(gq_attn_merge_kernel, dim3((unsigned)a.T, (unsigned)a.H), dim3(256), 0, st, a, (int)splits);
     return hipGetLastError();
 }
 
@@ -451,12 +488,13 @@ hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st) {
     if (a.T >= GQ_TILE_MIN_ROWS && (a.dim & 3) == 0 && (a.vdim & 3) == 0 && (a.ld_q & 3) == 0 && (a.ld_out & 3) == 0 && al16(a.q) && al16(a.out) && al16(a.cache)) {
         if (a.vdim <= 64) return launch_gq_attn_tile<1>(a, st);
         if (a.vdim <= 128) return launch_gq_attn_tile<2>(a, st);
-        return launch_gq_attn_tile<4>(a, st);
-    }
+        if (a.vdim <= 256) return launch_gq_attn_tile<4>(a, st);
+    }                                                            // (wider value heads: the per-row kernel below)
     const int Dm = a.dim > a.vdim ? a.dim : a.vdim;
     if (Dm <= 64) return launch_gq_attn_nj<1>(a, st);
     if (Dm <= 128) return launch_gq_attn_nj<2>(a, st);
-    return launch_gq_attn_nj<4>(a, st);
+    if (Dm <= 256) return launch_gq_attn_nj<4>(a, st);
+    return launch_gq_attn_nj<8>(a, st);
 }
 
 }  // namespace mi355

@@ -315,12 +315,15 @@ struct GqAttnArgs {
     int window;                            // cells at distance 0 .. window - 1 are seen; 0 = every earlier cell
     const float *sink;                     // [H] or nullptr: a logit without key or value in the softmax denominator
     const float *gate; int ld_gate;        // nullable: head h's output is multiplied by sigmoid(gate[t * ld_gate + h])
-    // steps of a few tokens: the scanned cells cut into `splits` runs, one workgroup each, merged afterwards; part: T * H * splits * (vdim + 2) floats
-    float *part; int splits;
+    // the scanned cells cut into runs, one workgroup each, merged afterwards: `splits` runs for steps of a few rows; for prompt batches with too few tiles
+    // to fill the device as many as n_kv_hint (the host's count of cells in use, 0: unknown) and the buffer allow.  part: room for part_floats floats,
+    // T * H * runs * (vdim + 2) are used
+    float *part; int splits; size_t part_floats; int n_kv_hint;
     // nullable, per token, host-made from the cell table: one past the highest cell that can hold a key of its sequence at or before its position, and the
     // lowest cell that can hold one still inside the window
     const int32_t *tok_hi, *tok_lo;
 };
+constexpr int GQ_TILE_MAX_SPLITS = 16;
 constexpr int GQ_TILE_MIN_ROWS = 32;     // batches from this many rows on take the LDS-tiled pass (64 rows x 64 cells per step) instead of one workgroup per (row, head)
 bool gq_attn_shape_ok(int H, int G, int dim, int vdim);
 hipError_t launch_gq_attn(const GqAttnArgs &a, hipStream_t st);

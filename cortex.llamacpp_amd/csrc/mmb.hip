@@ -372,7 +372,9 @@ hipError_t launch_mmb(const MMBArgs &a, hipStream_t st) {
     }
     if (!a.f32 && vec && (a.K % 16) == 0) {
         const dim3 big((unsigned)((a.N + 127) / 128), (unsigned)((rows_max + 127) / 128), (unsigned)a.nz);
-        if (big.x * big.y * big.z >= 512 && !gated) hipLaunchKernelGGL((mmb_mfma_kernel<2, false>), big, dim3(256), 0, st, a);
+        // (a grouped batch sizes its grid for the most rows ONE expert could hold; what counts for filling the device is the rows an expert holds on average)
+        const unsigned rows_avg = a.meta ? (unsigned)((a.T + a.nz - 1) / a.nz) : (unsigned)rows_max;
+        if (big.x * ((rows_avg + 127) / 128) * big.z >= (a.meta ? 256u : 512u) && !gated) hipLaunchKernelGGL((mmb_mfma_kernel<2, false>), big, dim3(256), 0, st, a);
         else {
             const dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((rows_max + 63) / 64), (unsigned)a.nz);
             if (gated) hipLaunchKernelGGL((mmb_mfma_kernel<1, true>), grid, dim3(256), 0, st, a);

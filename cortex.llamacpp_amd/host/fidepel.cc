@@ -57,7 +57,7 @@ Model *fidepel_build(const Json &cfg, const std::string &dir, Bf16Loader &ld, st
         if (!cfg_positive(err, "mixer.heads", L.heads, 4096) || !cfg_positive(err, "mixer.kv_heads", L.kv_heads, L.heads) || !cfg_positive(err, "mixer.dim", L.dim, 1 << 16) ||
             !cfg_positive(err, "mixer.vdim", L.vdim, 1 << 16)) return nullptr;
         if (L.heads % L.kv_heads != 0) { err = "configuration: mixer.heads must be a multiple of mixer.kv_heads"; return nullptr; }
-        if (!gq_attn_shape_ok(L.heads, L.kv_heads, L.dim, L.vdim)) { err = "attention: dim " + std::to_string(L.dim) + " / vdim " + std::to_string(L.vdim) + " is beyond what the attention kernel holds per lane (256)"; return nullptr; }
+        if (!gq_attn_shape_ok(L.heads, L.kv_heads, L.dim, L.vdim)) { err = "attention: dim " + std::to_string(L.dim) + " / vdim " + std::to_string(L.vdim) + " is beyond what the attention kernel holds per lane (512)"; return nullptr; }
         const int H = L.heads, G = L.kv_heads;
         L.scale = (float)mx["scale"].as_double(1.0);
         const Json &mask = mx["mask"];
@@ -180,7 +180,8 @@ hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, const f
     aa.window = L.window; aa.sink = nullptr; aa.gate = L.off_gate >= 0 ? nvx_a_ + L.off_gate : nullptr; aa.ld_gate = LD_P;
     aa.tok_hi = d_seg_ + 3 * (size_t)cp.n_ubatch;
     aa.tok_lo = M.max_window > 0 ? d_seg_ + 4 * (size_t)cp.n_ubatch : nullptr;
-    if (nvx_part_ && (long long)T * H <= LATENT_ATTN_SPLIT_MAX_PAIRS) { aa.part = nvx_part_; aa.splits = LATENT_ATTN_SPLITS; }
+    aa.part = nvx_part_; aa.part_floats = nvx_part_floats_; aa.n_kv_hint = n_kv_;
+    aa.splits = (long long)T * H <= LATENT_ATTN_SPLIT_MAX_PAIRS ? LATENT_ATTN_SPLITS : 1;
     FDP_TRY(launch_gq_attn(aa, stream_));
     FDP_TRY(nvx_linear(L.o, nvx_att_, H * L.vdim, T, nvx_y_, W));
     prof_mark("gq_attention");

@@ -302,7 +302,11 @@ bool Context::init_novorax(std::string &err) {
     {
         int kr = 1;                                              // widest record of a split attention scan: the latent, or a value head
         for (const NvxLayer &L : M.layers) kr = std::max(kr, L.type == NVX_LATENT ? L.kv_rank : L.type == NVX_GQ ? L.vdim : 1);
-        nvx_part_ = (float *)dalloc((size_t)LATENT_ATTN_SPLIT_MAX_PAIRS * LATENT_ATTN_SPLITS * (size_t)(kr + 2) * 4);
+        nvx_part_floats_ = (size_t)LATENT_ATTN_SPLIT_MAX_PAIRS * LATENT_ATTN_SPLITS * (size_t)(kr + 2);
+        // grouped-query layers also cut the block chains of short prompt batches: records for up to 1024 rows x 4 runs of the widest layer
+        for (const NvxLayer &L : M.layers)
+            if (L.type == NVX_GQ) nvx_part_floats_ = std::max(nvx_part_floats_, std::min<size_t>(T, 1024) * (size_t)L.heads * 4 * (size_t)(L.vdim + 2));
+        nvx_part_ = (float *)dalloc(nvx_part_floats_ * 4);
     }
     if (!x_ || !xn_ || !xo_ || !nvx_x0_ || !nvx_xcat_ || !nvx_y_ || !nvx_a_ || !nvx_cq_ || !nvx_q_ || !nvx_qa_ || !nvx_lat_ || !nvx_att_ || !nvx_o_ || !nvx_ff_) { err = "activation buffer allocation failed"; return false; }
     if (M.max_top > 0) {

@@ -197,7 +197,8 @@ class Context {
     std::vector<float *> nvx_S_, nvx_n_, nvx_m_;            // [mlstm run] [n_seq_max][H][D][VD], [..][H][D], [..][H]
     std::vector<uint64_t> nvx_seq_len_;                     // tokens every sequence id has been fed (the recurrent state cannot be cut back)
     float *nvx_x0_ = nullptr, *nvx_xcat_ = nullptr, *nvx_y_ = nullptr, *nvx_a_ = nullptr, *nvx_cq_ = nullptr, *nvx_q_ = nullptr, *nvx_qa_ = nullptr, *nvx_lat_ = nullptr;
-    float *nvx_part_ = nullptr;                             // split records of the latent attention of single-token steps
+    float *nvx_part_ = nullptr;                             // records of attention scans that were cut into runs (single-token steps; short prompt batches)
+    size_t nvx_part_floats_ = 0;
     float *nvx_att_ = nullptr, *nvx_o_ = nullptr, *nvx_ff_ = nullptr, *nvx_xg_ = nullptr, *nvx_yg_ = nullptr;
     int32_t *nvx_ids_ = nullptr, *nvx_meta_ = nullptr, *nvx_slot_ = nullptr, *nvx_tokof_ = nullptr;
     int32_t *h_seg_ = nullptr, *d_seg_ = nullptr;           // [5][n_ubatch]: start, length, slot of every segment; upper and lower scan bound of every token

@@ -339,6 +339,7 @@ def test_window_edges_while_other_requests_come_and_go(pkg, tmp_path):
                       loop=(0, 1, 1), residual_mult=1.0)),
     ("wide_heads", S.config([S.attention(heads=4, kv_heads=2, dim=160, vdim=72, window=33, rot_dims=64, mlp=S.moe(n=7, top=3, ff=56, groups=None, shared=80))], width=136, vocab=301)),
     ("wide_values", S.config([S.attention(heads=2, kv_heads=1, dim=32, vdim=256, window=40, rot_dims=32, mlp=None)], width=64, vocab=77)),
+    ("very_wide_heads", S.config([S.attention(heads=2, kv_heads=1, dim=320, vdim=272, window=50, rot_dims=320, mlp=None)], width=96, vocab=55)),
     ("equal_head_sizes", S.config([S.attention(heads=8, kv_heads=4, dim=64, vdim=64, window=16, rot_dims=32, mlp=S.moe(n=16, top=4, ff=32, groups=(8, 4), shared=32))], width=128, vocab=200)),
     # heads whose keys and values do not start on 16-byte boundaries (the attention kernel's scalar-load form), a width that is no multiple of 8
     ("unaligned", S.config([S.attention(heads=3, kv_heads=3, dim=10, vdim=14, window=6, rot_dims=6, mlp=S.moe(n=4, top=2, ff=30, groups=(2, 1), shared=18))], width=44, vocab=29)),
