@@ -41,11 +41,11 @@ SIZES = {
 
 def config_of(s: FidepelSize) -> dict:
     mixer = {"dim": s.dim, "heads": s.heads, "kv_heads": s.kv_heads, "mask": {"size": s.window},
-             "rot": {"base": 500000.0, "dims": s.rot_dims, "scaling": {"factor": 8.0}}, "scale": float(s.dim ** -0.5), "vdim": s.vdim}
+             "rot": {"base": 500000.0, "dims": s.rot_dims, "scaling": {"factor": 4.0}}, "scale": float(s.dim ** -0.5), "vdim": s.vdim}
     mlp = {"kind": "moe", "expert": {"ff": s.expert_ff},
-           "router": {"experts": s.n_expert, "groups": {"count": s.groups[0], "keep": s.groups[1]}, "scale": 2.0, "top": s.top}, "shared": {"ff": s.shared_ff}}
+           "router": {"experts": s.n_expert, "groups": {"count": s.groups[0], "keep": s.groups[1]}, "scale": 1.5, "top": s.top}, "shared": {"ff": s.shared_ff}}
     cfg = {"architecture": "Fidepel", "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp} for _ in range(s.n_layer)],
-           "norm": {"eps": 1e-6}, "residual_mult": 0.7, "vocab": s.vocab, "width": s.width}
+           "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": s.vocab, "width": s.width}
     if s.loop:
         cfg["loop"] = {"start": s.loop[0], "stop": s.loop[1], "times": s.loop[2]}
     return cfg
