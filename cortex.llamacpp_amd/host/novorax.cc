@@ -1,6 +1,8 @@
-// novorax.cc — loading a Novorax folder and running its layer stack inside Context (see novorax.h for the design, runtime.h for the context).
+// novorax.cc — the folder models (config.json + model.safetensors): the registry that picks a design's loader by "architecture", the Novorax loader, and what
+// every such design shares inside Context - buffers, cache planes and state slots, segment lists and scan bounds, the layer-run loop, the output head
+// (novorax.h describes the designs, runtime.h the context; the Fidepel loader and its block are in fidepel.cc).
 //
-// The context's own machinery carries it: the cell table (find / free / sequence masks) addresses the latent-attention cache planes, the micro-batch staging
+// The context's own machinery carries them: the cell table (find / free / sequence masks) addresses the attention layers' cache planes, the micro-batch staging
 // block brings tokens, positions, cells and sequence ids to the device, the sequence id is the slot of the recurrent state, logits / arg-max / top-k leave
 // through the usual buffers.  What is new per micro-batch is the list of segments (runs of consecutive rows of one sequence) the recurrence walks.
 #include <sys/stat.h>
