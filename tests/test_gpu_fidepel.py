@@ -455,3 +455,58 @@ def test_trace_replay_tool(full, tmp_path):
         g1 = np.fromfile(out / "1.f32", "<f4").reshape(-1, V)
         g2 = np.fromfile(out / "2.f32", "<f4").reshape(-1, V)
         assert row_err(g0, ra[[0, 9]]) <= tol and row_err(g1, rb[[8]]) <= tol and row_err(g2, ra[[20, 12]]) <= tol
+
+
+def test_trace_tool_with_a_pool_that_is_always_full(pkg, tmp_path):
+    """Up to four live requests of unequal lengths fed in portions of changing size beside single tokens of the others, in a pool that holds exactly what
+    the live requests need (each rounded up to 64 cells): a finished request's cells and slot go to the next one at once.  Every position of every request
+    is asked for and compared with the restatement, in both precisions."""
+    cfg = S.config([S.attention(heads=6, kv_heads=3, dim=16, vdim=24, window=21, rot_dims=12, mlp=S.moe(n=9, top=2, ff=24, groups=(3, 2), shared=40)),
+                    S.attention(heads=2, kv_heads=1, dim=32, vdim=16, window=70, rot_dims=32, factor=2.0, mlp=S.moe(n=4, top=1, ff=32, groups=None, shared=0)),
+                    S.attention(heads=4, kv_heads=4, dim=8, vdim=8, window=0, rot_dims=0, mlp=None)], width=88, vocab=211, loop=(0, 2, 2))
+    rig = Rig(pkg, tmp_path / "pool", cfg, seed=31)
+    V = cfg["vocab"]
+    rng = np.random.default_rng(5)
+    lengths = [150, 64, 97, 1, 33, 128, 70, 191, 2, 65]
+    reqs = {f"q{i}": toks(n, V, 300 + i) for i, n in enumerate(lengths)}
+    waiting, live, at = list(reqs), [], {}
+    steps, need = [], 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            r = waiting.pop(0)
+            live.append(r)
+            at[r] = 0
+        need = max(need, sum((len(reqs[r]) + 63) // 64 * 64 for r in live))
+        entries, end = [], []
+        for k, r in enumerate(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                         # a request may sit a step out
+            n = int(rng.choice([1, 1, 1, 2, 3, 5, 17, 40])) if at[r] > 0 or k != 1 else len(reqs[r])
+            n = min(n, len(reqs[r]) - at[r])
+            entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == len(reqs[r]):
+                end.append(r)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+        live = [r for r in live if r not in end]
+    want = {r: rig.ref(t) for r, t in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / dtype
+        p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", rig.dir, "--dtype", dtype, "--out", str(out), "--max-tokens", str(need)],
+                           input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+        assert p.returncode == 0, p.stderr[-2000:]
+        got, fed = {r: [] for r in reqs}, {r: 0 for r in reqs}
+        for st in steps:
+            if not any(e["want"] for e in st["entries"]):
+                continue
+            rows = np.fromfile(out / f"{st['step']}.f32", "<f4").reshape(-1, V)
+            k = 0
+            for e in st["entries"]:
+                got[e["id"]].append(rows[k:k + len(e["want"])])
+                k += len(e["want"])
+            assert k == len(rows)
+        errs = np.concatenate([row_errs(np.concatenate(got[r]), want[r]) for r in reqs])
+        if dtype == "float32":
+            assert errs.max() <= F32_TOL, errs.max()
+        else:
+            assert np.median(errs) <= 2e-2 and np.percentile(errs, 90) <= BF16_TOL, (np.median(errs), np.percentile(errs, 90), errs.max())
