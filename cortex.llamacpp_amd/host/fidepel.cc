@@ -161,13 +161,11 @@ static bool routed_as_groups(const NvxLayer &L, int T) {
     return L.ff_kind == NVX_FF_ROUTED && T * L.top > 32 && L.n_expert <= 64 && (size_t)T * L.top * 4 <= 60 * 1024;
 }
 
-// h: the rows every sublayer reads - the normed stream (pn == nullptr), or the stream itself with the norm weight pn for the launches that norm their few
-// rows on the way in
-hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, const float *h, const float *pn, int T) {
+// behind the block projection (nvx_a_): queries prepared, keys and values stored, attention, output projection -> nvx_y_
+hipError_t Context::nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T) {
     const NovoraxModel &M = *model->nvx;
     const int W = M.width, H = L.heads, G = L.kv_heads, LD_P = L.proj.N;
     float *cache = nvx_cache_[(size_t)r.plane];
-    FDP_TRY(nvx_linear(L.proj, h, W, T, nvx_a_, LD_P, MMB_STORE, nullptr, 1.0f, pn));
     GqPrepArgs pa{};
     pa.p = nvx_a_; pa.ld_p = LD_P; pa.T = T; pa.H = H; pa.G = G; pa.dim = L.dim; pa.vdim = L.vdim;
     pa.wq_norm = L.q_norm; pa.wk_norm = L.k_norm; pa.eps = M.eps; pa.rot_dims = L.rot_dims; pa.rot_freq = L.rot_freq;
@@ -214,11 +212,15 @@ hipError_t Context::nvx_routed_experts(const NvxLayer &L, const float *h, const 
     }
     FDP_TRY(launch_mmb(u, stream_));
     FDP_TRY(launch_mmb(d, stream_));
-    if (L.shared_ff > 0) {
-        FDP_TRY(nvx_linear(L.s_up, h, W, T, nvx_sh_, L.shared_ff, MMB_RELU2, nullptr, 1.0f, pn));
-        FDP_TRY(nvx_linear(L.s_down, nvx_sh_, L.shared_ff, T, nvx_ys_, W));
-    }
     prof_mark("routed_experts");
+    return hipSuccess;
+}
+
+hipError_t Context::nvx_shared_expert(const NvxLayer &L, const float *h, const float *pn, int T) {
+    const int W = model->nvx->width;
+    FDP_TRY(nvx_linear(L.s_up, h, W, T, nvx_sh_, L.shared_ff, MMB_RELU2, nullptr, 1.0f, pn));
+    FDP_TRY(nvx_linear(L.s_down, nvx_sh_, L.shared_ff, T, nvx_ys_, W));
+    prof_mark("shared_expert");
     return hipSuccess;
 }
 
@@ -235,11 +237,39 @@ hipError_t Context::nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T
         h = xn_; pn = nullptr;
     }
     if (L.type != NVX_GQ) return hipErrorInvalidValue;
-    FDP_TRY(nvx_gq_attention(L, r, h, pn, T));
-    const bool routed = L.ff_kind == NVX_FF_ROUTED;
-    if (routed) FDP_TRY(nvx_routed_experts(L, h, pn, T));
-    else if (L.ff_kind != NVX_FF_NONE) return hipErrorInvalidValue;
-    FDP_TRY(launch_block_combine(x_, nvx_y_, routed && L.shared_ff > 0 ? nvx_ys_ : nullptr, nvx_yg_, nvx_rw_, routed && grouped ? nvx_slot_ : nullptr, T, W,
+    const bool routed = L.ff_kind == NVX_FF_ROUTED, shared = routed && L.shared_ff > 0;
+    if (!routed && L.ff_kind != NVX_FF_NONE) return hipErrorInvalidValue;
+    // h: the rows every sublayer reads - the normed stream (pn == nullptr), or the stream itself with the norm weight pn for the launches that norm their
+    // few rows on the way in.  One projection [q ; k ; v ; g ; router] for all of them
+    FDP_TRY(nvx_linear(L.proj, h, W, T, nvx_a_, L.proj.N, MMB_STORE, nullptr, 1.0f, pn));
+    // behind it the attention, the routed experts and the shared expert touch no buffer of each other until the closing sum: the two feed-forward branches
+    // go to side streams (events only order them; a profile run keeps one stream so that its marks bracket whole sublayers)
+    const bool fork = nvx_fork_ok_ && routed && !profile_;
+    hipStream_t const main_stream = stream_;
+    struct Back { hipStream_t &s; hipStream_t v; ~Back() { s = v; } } back{stream_, main_stream};   // (every helper launches on stream_)
+    if (fork) {
+        FDP_TRY(hipEventRecord(nvx_fork_ev_, main_stream));
+        FDP_TRY(hipStreamWaitEvent(nvx_side_[0], nvx_fork_ev_, 0));
+        stream_ = nvx_side_[0];
+        FDP_TRY(nvx_routed_experts(L, h, pn, T));
+        FDP_TRY(hipEventRecord(nvx_join_ev_[0], nvx_side_[0]));
+        if (shared) {
+            FDP_TRY(hipStreamWaitEvent(nvx_side_[1], nvx_fork_ev_, 0));
+            stream_ = nvx_side_[1];
+            FDP_TRY(nvx_shared_expert(L, h, pn, T));
+            FDP_TRY(hipEventRecord(nvx_join_ev_[1], nvx_side_[1]));
+        }
+        stream_ = main_stream;
+    }
+    FDP_TRY(nvx_gq_attention(L, r, T));
+    if (fork) {
+        FDP_TRY(hipStreamWaitEvent(main_stream, nvx_join_ev_[0], 0));
+        if (shared) FDP_TRY(hipStreamWaitEvent(main_stream, nvx_join_ev_[1], 0));
+    } else if (routed) {
+        FDP_TRY(nvx_routed_experts(L, h, pn, T));
+        if (shared) FDP_TRY(nvx_shared_expert(L, h, pn, T));
+    }
+    FDP_TRY(launch_block_combine(x_, nvx_y_, shared ? nvx_ys_ : nullptr, nvx_yg_, nvx_rw_, routed && grouped ? nvx_slot_ : nullptr, T, W,
                                  routed ? L.top : 0, M.residual_mult, stream_));
     return hipSuccess;
 }

@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <sstream>
@@ -325,6 +326,15 @@ bool Context::init_novorax(std::string &err) {
         nvx_sh_ = (float *)dalloc(T * (size_t)M.max_shared_ff * 4);
         nvx_ys_ = (float *)dalloc(T * W * 4);
         if (!nvx_sh_ || !nvx_ys_) { err = "shared expert buffers allocation failed"; return false; }
+    }
+    if (M.parallel_block) {
+        // side streams of the block's feed-forward branches (default priority, like the main one); MI355_BLOCK_FORK=0 keeps every launch on the main stream
+        const char *ev = getenv("MI355_BLOCK_FORK");
+        nvx_fork_ok_ = !(ev && ev[0] == '0');
+        for (int i = 0; i < 2 && nvx_fork_ok_; i++)
+            nvx_fork_ok_ = hipStreamCreateWithFlags(&nvx_side_[i], hipStreamNonBlocking) == hipSuccess &&
+                           hipEventCreateWithFlags(&nvx_join_ev_[i], hipEventDisableTiming) == hipSuccess;
+        nvx_fork_ok_ = nvx_fork_ok_ && hipEventCreateWithFlags(&nvx_fork_ev_, hipEventDisableTiming) == hipSuccess;
     }
     d_argmax_ = (int32_t *)dalloc(T * 4);
     argmax_scratch_ = (float *)dalloc(T * 129 * 4);

@@ -549,6 +549,9 @@ Context::~Context() {
     if (d_topk_adj_) (void)hipFree(d_topk_adj_);
     if (topk_scratch_) { (void)hipFree(topk_scratch_); topk_scratch_ = nullptr; }
     if (h_moe_meta_) (void)hipHostFree(h_moe_meta_);
+    for (hipStream_t &sd : nvx_side_) if (sd) (void)hipStreamDestroy(sd);
+    if (nvx_fork_ev_) (void)hipEventDestroy(nvx_fork_ev_);
+    for (hipEvent_t &ev : nvx_join_ev_) if (ev) (void)hipEventDestroy(ev);
     if (stream_) (void)hipStreamDestroy(stream_);
 }
 

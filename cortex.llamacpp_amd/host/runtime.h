@@ -186,9 +186,15 @@ class Context {
     hipError_t nvx_feed_forward(const NvxLayer &L, int T);
     // fidepel.cc: a block whose mixer and feed-forward read one norm; grouped-query attention on the run's cache plane; experts picked by a router
     hipError_t nvx_parallel_block(const NvxLayer &L, const NvxRun &r, int T);
-    hipError_t nvx_gq_attention(const NvxLayer &L, const NvxRun &r, const float *h, const float *pn, int T);
+    hipError_t nvx_gq_attention(const NvxLayer &L, const NvxRun &r, int T);
     hipError_t nvx_routed_experts(const NvxLayer &L, const float *h, const float *pn, int T);
+    hipError_t nvx_shared_expert(const NvxLayer &L, const float *h, const float *pn, int T);
     float *nvx_sh_ = nullptr, *nvx_ys_ = nullptr, *nvx_rw_ = nullptr;   // shared expert's hidden rows and output; router weights [T][top]
+    // the three readers of a one-norm block's projection - attention, routed experts, shared expert - are independent until the block's closing sum: the two
+    // feed-forward branches run on side streams forked behind the projection and joined in front of the sum (eagerly and inside the captured step alike)
+    hipStream_t nvx_side_[2] = {nullptr, nullptr};
+    hipEvent_t nvx_fork_ev_ = nullptr, nvx_join_ev_[2] = {nullptr, nullptr};
+    bool nvx_fork_ok_ = false;
     // runs of consecutive tokens of one sequence -> segment arrays; per-token scan bounds of the attention (pinned, then device)
     bool nvx_stage_segments(int n, const int32_t *seq, const int32_t *pos, const int *tcell);
     void nvx_state_reset(int seq);                          // seq < 0: every slot

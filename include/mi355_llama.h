@@ -75,7 +75,7 @@ typedef struct mi355_model_params {
 
 MI355_API mi355_model_params mi355_model_default_params(void);
 /* common_init_from_params -> llama_model_load_from_file (llama_server_context.cc:207) */
-/* path: a GGUF file, or a folder holding config.json + model.safetensors (architecture "Novorax") */
+/* path: a GGUF file, or a folder holding config.json + model.safetensors (architecture "Novorax" or "Fidepel") */
 MI355_API mi355_model *mi355_model_load_from_file(const char *path_gguf, mi355_model_params params);
 MI355_API void         mi355_model_free(mi355_model *model);
 

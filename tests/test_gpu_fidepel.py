@@ -400,6 +400,20 @@ def test_graph_replays_equal_eager_steps(full):
     assert row_err(outs[0], full.ref(t)[8:]) <= F32_TOL
 
 
+def test_feed_forward_branches_on_side_streams_change_no_bit(full, monkeypatch):
+    """The routed and the shared experts of a block run on side streams beside its attention (forked behind the block projection, joined before the closing
+    sum); MI355_BLOCK_FORK=0 keeps every launch on one stream.  Same launches, same order of additions: prompts, portions and replayed single-token steps
+    give the same bits either way."""
+    t = toks(90, full.cfg["vocab"], 33)
+    outs = []
+    for fork in ("1", "0"):
+        monkeypatch.setenv("MI355_BLOCK_FORK", fork)
+        c = full.ctx(n_ubatch=32)
+        outs.append(np.concatenate([feed_in_portions(c, t[:60], [40, 3, 17]), one_by_one(c, t, 60)]))
+    assert np.array_equal(outs[0], outs[1])
+    assert row_err(outs[0], full.ref(t)) <= F32_TOL
+
+
 # ------------------------------------------------------------------------------------------ the engine and the tools
 def test_greedy_generation_through_the_engine(pkg, full):
     """loadmodel -> chat completion through the slot scheduler, two requests side by side; the text is decimal token ids."""
